@@ -1,0 +1,94 @@
+/*
+** Internal C++ interface between the C-ABI entry points and the gfx950 kernels
+** of the optimizer step.  Not installed; the public surface is the headers under include/.
+**
+** Work decomposition.  The flat of n elements is cut into tiles of kTile
+** elements counted from the start of the flat (not from the start of a
+** tensor), so vector accesses are aligned whenever the flat's base pointers
+** are.  A launch table maps each tile to the tensor that holds its first
+** element; a tile that lies wholly inside one tensor runs the 16-byte vector
+** path with that tensor's attributes held in scalars, a tile that crosses a
+** tensor boundary (or the ragged end of the flat) runs an element-wise path
+** that looks the tensor up per element.  One launch therefore covers every
+** tensor, however small, and the long tail of bias / LayerNorm vectors costs
+** no extra launches.
+*/
+#ifndef ANNI_ADAM_KERNELS_H__
+#define ANNI_ADAM_KERNELS_H__
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "adam_math.h"
+
+namespace anni {
+
+enum { kF32 = 0, kBF16 = 1, kFP8 = 2 };
+
+constexpr int kThreads = 256;			/* four 64-lane wavefronts */
+constexpr int kQuad = 4;			/* elements per lane per access */
+constexpr int kTile = 4096;			/* elements per tile */
+constexpr int kQuadsPerTile = kTile / (kThreads * kQuad);	/* 4 */
+constexpr int kMaxPartials = 8192;		/* upper bound on the sum-of-squares grid */
+
+constexpr uint32_t kSegDecay = 1u;		/* decoupled weight decay applies */
+constexpr uint32_t kSegTwin = 2u;		/* bf16 twin is written */
+
+/* One tensor of the flat: elements [begin, end). */
+struct Seg {
+	int64_t		begin;
+	int64_t		end;
+	uint32_t	flags;
+	uint32_t	pad;
+};
+
+/* Written by the step on the device; read back only when the host asks. */
+struct StepState {
+	double	sumsq;
+	double	norm;
+	double	grad_scale;	/* after the clip factor */
+	int	skipped;
+	int	clipped;
+};
+
+/* The arrays and launch table one launch works on (all device pointers). */
+struct Flat {
+	float		*p;
+	void		*g;
+	void		*m;
+	void		*v;
+	uint16_t	*twin;		/* may be NULL */
+	int64_t		n;
+	int		grad_type;
+	int		moment_type;
+	const Seg	*segs;		/* NULL: one tensor with uniform_flags */
+	const int32_t	*tile_seg;	/* NULL when segs is NULL */
+	const float	*gscale;	/* per-tensor dequant scale (fp8 gradients) */
+	uint32_t	uniform_flags;
+};
+
+/* How the update obtains the global norm (use_norm == 0: grad_scale is final). */
+struct NormIn {
+	int		use_norm;
+	const double	*partials;
+	int		n_partials;
+	double		clip;
+	int		skip_nonfinite;
+	StepState	*state;		/* may be NULL */
+};
+
+/* Number of persistent workgroups for a flat of n elements on the current device. */
+int	grid_for(int64_t n);
+
+/* partials[0..*n_partials) = per-workgroup sums of (g * grad_scale)^2, fixed order. */
+int	launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *partials,
+		int *n_partials);
+/* state = {sum, sqrt, clip-adjusted scale, flags} from the partials, fixed order. */
+int	launch_finalize(hipStream_t st, const double *partials, int n_partials, double clip,
+		int skip_nonfinite, double grad_scale, StepState *state);
+int	launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double grad_scale,
+		const NormIn &norm);
+int	launch_f32_to_bf16(hipStream_t st, uint16_t *dst, const float *src, int64_t n);
+int	launch_fill_bytes(hipStream_t st, void *dst, int value, size_t nbytes);
+
+} /* namespace anni */
+#endif

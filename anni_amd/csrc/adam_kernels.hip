@@ -1,0 +1,695 @@
+/*
+** gfx950 kernels of the AnnI optimizer step: the global sum of squares (clip
+** norm), the fused AdamW update with bf16 twin emission, and the small helpers
+** around them.  Everything here is a memory-bound stream: 64-lane wavefronts,
+** 16-byte accesses per lane where the element type allows, persistent
+** workgroups striding over tiles, no matrix cores.
+**
+** Replaces (does not port) the reference's device step, num/gpu_cuda.cu:8417-8712:
+** the arithmetic follows the reference's HOST loop (lang/lm_adam.c:571-598) in
+** double, see adam_math.h.
+*/
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include "adam_kernels.h"
+
+namespace anni {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+/* ---- typed quad access ------------------------------------------------- */
+
+template <bool NT, typename T>
+__device__ __forceinline__ T ld(const T *p)
+{
+	if (NT)
+		return __builtin_nontemporal_load(p);
+	return *p;
+}
+
+template <bool NT, typename T>
+__device__ __forceinline__ void st(T *p, T v)
+{
+	if (NT)
+		__builtin_nontemporal_store(v, p);
+	else
+		*p = v;
+}
+
+/* Four consecutive values of a typed array, starting at element i (i % 4 == 0), as floats. */
+template <int T, bool NT>
+__device__ __forceinline__ f32x4 load_quad(const void *base, int64_t i, float scale)
+{
+	f32x4 r;
+
+	if (T == kF32) {
+		r = ld<NT>((const f32x4 *)((const float *)base + i));
+	} else if (T == kBF16) {
+		const u32x2 w = ld<NT>((const u32x2 *)((const uint16_t *)base + i));
+
+		r.x = __uint_as_float(w.x << 16);
+		r.y = __uint_as_float(w.x & 0xffff0000u);
+		r.z = __uint_as_float(w.y << 16);
+		r.w = __uint_as_float(w.y & 0xffff0000u);
+	} else {
+		const uint32_t w = ld<NT>((const uint32_t *)((const uint8_t *)base + i));
+
+		r.x = fp8_e4m3_decode(w & 0xffu) * scale;
+		r.y = fp8_e4m3_decode((w >> 8) & 0xffu) * scale;
+		r.z = fp8_e4m3_decode((w >> 16) & 0xffu) * scale;
+		r.w = fp8_e4m3_decode(w >> 24) * scale;
+	}
+	return r;
+}
+
+/* Stores four floats into an f32 or bf16 array (bf16: round to nearest even). */
+template <int T, bool NT>
+__device__ __forceinline__ void store_quad(void *base, int64_t i, f32x4 x)
+{
+	if (T == kF32) {
+		st<NT>((f32x4 *)((float *)base + i), x);
+	} else {
+		u32x2 w;
+
+		w.x = bf16_rne(x.x) | (bf16_rne(x.y) << 16);
+		w.y = bf16_rne(x.z) | (bf16_rne(x.w) << 16);
+		st<NT>((u32x2 *)((uint16_t *)base + i), w);
+	}
+}
+
+template <int T, bool NT>
+__device__ __forceinline__ void zero_quad(void *base, int64_t i)
+{
+	if (T == kF32) {
+		const f32x4 z = {0.0f, 0.0f, 0.0f, 0.0f};
+
+		st<NT>((f32x4 *)((float *)base + i), z);
+	} else if (T == kBF16) {
+		const u32x2 z = {0u, 0u};
+
+		st<NT>((u32x2 *)((uint16_t *)base + i), z);
+	} else {
+		st<NT>((uint32_t *)((uint8_t *)base + i), 0u);
+	}
+}
+
+template <int T>
+__device__ __forceinline__ float load_one(const void *base, int64_t i, float scale)
+{
+	if (T == kF32)
+		return ((const float *)base)[i];
+	if (T == kBF16)
+		return bf16_widen(((const uint16_t *)base)[i]);
+	return fp8_e4m3_decode(((const uint8_t *)base)[i]) * scale;
+}
+
+template <int T>
+__device__ __forceinline__ void store_one(void *base, int64_t i, float x)
+{
+	if (T == kF32)
+		((float *)base)[i] = x;
+	else
+		((uint16_t *)base)[i] = (uint16_t)bf16_rne(x);
+}
+
+template <int T>
+__device__ __forceinline__ void zero_one(void *base, int64_t i)
+{
+	if (T == kF32)
+		((float *)base)[i] = 0.0f;
+	else if (T == kBF16)
+		((uint16_t *)base)[i] = 0;
+	else
+		((uint8_t *)base)[i] = 0;
+}
+
+/* ---- reductions --------------------------------------------------------- */
+
+/*
+** Sum over the 256 lanes of a workgroup in a fixed tree: shuffles inside each
+** 64-lane wavefront, then the four wavefront sums through LDS in index order.
+** Every lane returns the same total.  lds must hold 4 doubles.
+*/
+__device__ __forceinline__ double block_sum(double x, double *lds)
+{
+	const int tid = threadIdx.x;
+
+#pragma unroll
+	for (int off = 32; off > 0; off >>= 1)
+		x += __shfl_down(x, off, 64);
+	if ((tid & 63) == 0)
+		lds[tid >> 6] = x;
+	__syncthreads();
+	const double total = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+	__syncthreads();
+	return total;
+}
+
+/* Second stage of the norm: the per-workgroup partials in index order, then block_sum. */
+__device__ __forceinline__ double partials_sum(const double *partials, int np, double *lds)
+{
+	double acc = 0.0;
+
+	for (int i = threadIdx.x; i < np; i += kThreads)
+		acc += partials[i];
+	return block_sum(acc, lds);
+}
+
+struct NormOut {
+	double	gs;
+	bool	skip;
+};
+
+/*
+** norm = sqrt(sum); a non-finite norm skips the step (lang/lm_adam.c:474-483);
+** norm > clip scales the gradients by clip / (norm + 1e-12) (lm_adam.c:581-585).
+*/
+__device__ __forceinline__ NormOut norm_decide(double ss, double clip, int skip_nonfinite,
+	double grad_scale, StepState *state, bool writer)
+{
+	NormOut o;
+	const double norm = sqrt(ss);
+	const bool bad = skip_nonfinite && !(fabs(norm) <= 1.7976931348623157e308);
+	const bool clipped = !bad && clip > 0.0 && norm > clip;
+
+	o.gs = grad_scale;
+	o.skip = bad;
+	if (clipped)
+		o.gs = grad_scale * (clip / (norm + 1e-12));
+	if (writer && state) {
+		state->sumsq = ss;
+		state->norm = norm;
+		state->grad_scale = o.gs;
+		state->skipped = bad ? 1 : 0;
+		state->clipped = clipped ? 1 : 0;
+	}
+	return o;
+}
+
+/* ---- sum of squares ------------------------------------------------------ */
+
+struct SumsqArgs {
+	const void	*g;
+	int64_t		n;
+	const Seg	*segs;
+	const int32_t	*tile_seg;
+	const float	*gscale;
+	double		grad_scale;
+	double		*partials;
+	int		vec_ok;
+};
+
+template <int GT, bool NT>
+__global__ __launch_bounds__(kThreads) void sumsq_kernel(SumsqArgs a)
+{
+	__shared__ double lds[4];
+	const int tid = threadIdx.x;
+	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
+	double acc0 = 0.0, acc1 = 0.0, acc2 = 0.0, acc3 = 0.0;
+
+	for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+		const int64_t base = tile * kTile;
+		const int64_t end = base + kTile < a.n ? base + kTile : a.n;
+		int s = a.tile_seg ? a.tile_seg[tile] : 0;
+		const int64_t seg_end = a.segs ? a.segs[s].end : a.n;
+
+		if (a.vec_ok && end - base == kTile && seg_end >= end) {
+			const float sc = (GT == kFP8) ? a.gscale[s] : 1.0f;
+			f32x4 G[kQuadsPerTile];
+
+#pragma unroll
+			for (int u = 0; u < kQuadsPerTile; u++)
+				G[u] = load_quad<GT, NT>(a.g, base + (int64_t)(u * kThreads + tid) * kQuad, sc);
+#pragma unroll
+			for (int u = 0; u < kQuadsPerTile; u++) {
+				const double x0 = (double)G[u].x * a.grad_scale;
+				const double x1 = (double)G[u].y * a.grad_scale;
+				const double x2 = (double)G[u].z * a.grad_scale;
+				const double x3 = (double)G[u].w * a.grad_scale;
+
+				acc0 += x0 * x0;
+				acc1 += x1 * x1;
+				acc2 += x2 * x2;
+				acc3 += x3 * x3;
+			}
+		} else {
+			for (int64_t i = base + tid; i < end; i += kThreads) {
+				float sc = 1.0f;
+
+				if (a.segs)
+					while (i >= a.segs[s].end)
+						s++;
+				if (GT == kFP8)
+					sc = a.gscale[s];
+				const double x = (double)load_one<GT>(a.g, i, sc) * a.grad_scale;
+
+				acc0 += x * x;
+			}
+		}
+	}
+	const double total = block_sum((acc0 + acc1) + (acc2 + acc3), lds);
+
+	if (tid == 0)
+		a.partials[blockIdx.x] = total;
+}
+
+struct FinalizeArgs {
+	const double	*partials;
+	int		n_partials;
+	double		clip;
+	int		skip_nonfinite;
+	double		grad_scale;
+	StepState	*state;
+};
+
+__global__ __launch_bounds__(kThreads) void finalize_kernel(FinalizeArgs a)
+{
+	__shared__ double lds[4];
+	const double ss = partials_sum(a.partials, a.n_partials, lds);
+
+	(void)norm_decide(ss, a.clip, a.skip_nonfinite, a.grad_scale, a.state,
+	    threadIdx.x == 0);
+}
+
+/* ---- the update ---------------------------------------------------------- */
+
+struct UpdateArgs {
+	float		*p;
+	void		*g;
+	void		*m;
+	void		*v;
+	uint16_t	*twin;
+	int64_t		n;
+	const Seg	*segs;
+	const int32_t	*tile_seg;
+	const float	*gscale;
+	uint32_t	uniform_flags;
+	int		vec_ok;
+	StepConsts	c;
+	double		grad_scale;
+	/* norm */
+	int		use_norm;
+	int		skip_nonfinite;
+	const double	*partials;
+	int		n_partials;
+	double		clip;
+	StepState	*state;
+};
+
+/* U = quads a lane keeps in flight at once (kQuadsPerTile % U == 0). */
+template <int GT, int MT, int U, bool NT>
+__global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
+{
+	__shared__ double lds[4];
+	const int tid = threadIdx.x;
+	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
+	double gs = a.grad_scale;
+	bool skip = false;
+
+	if (a.use_norm) {
+		/*
+		** Every workgroup folds the same partials in the same order, so all of
+		** them derive the same scale without any cross-workgroup handshake.
+		*/
+		const double ss = partials_sum(a.partials, a.n_partials, lds);
+		const NormOut o = norm_decide(ss, a.clip, a.skip_nonfinite, gs, a.state,
+		    blockIdx.x == 0 && tid == 0);
+
+		gs = o.gs;
+		skip = o.skip;
+	}
+	for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+		const int64_t base = tile * kTile;
+		const int64_t end = base + kTile < a.n ? base + kTile : a.n;
+		int s = a.tile_seg ? a.tile_seg[tile] : 0;
+		const int64_t seg_end = a.segs ? a.segs[s].end : a.n;
+		const bool whole = a.vec_ok && end - base == kTile;
+
+		if (skip) {
+			/* Non-finite norm: p, m, v and the twins stay as they are; gradients are cleared. */
+			if (whole) {
+#pragma unroll
+				for (int u = 0; u < kQuadsPerTile; u++)
+					zero_quad<GT, NT>(a.g, base + (int64_t)(u * kThreads + tid) * kQuad);
+			} else {
+				for (int64_t i = base + tid; i < end; i += kThreads)
+					zero_one<GT>(a.g, i);
+			}
+			continue;
+		}
+		if (whole && seg_end >= end) {
+			const uint32_t flags = a.segs ? a.segs[s].flags : a.uniform_flags;
+			const bool decay = a.c.decay_on && (flags & kSegDecay) != 0;
+			const bool twin = (flags & kSegTwin) != 0 && a.twin != nullptr;
+			const float sc = (GT == kFP8) ? a.gscale[s] : 1.0f;
+
+#pragma unroll
+			for (int sub = 0; sub < kQuadsPerTile / U; sub++) {
+				f32x4 P[U], G[U], M[U], V[U];
+				int64_t idx[U];
+
+#pragma unroll
+				for (int u = 0; u < U; u++) {
+					idx[u] = base + (int64_t)((sub * U + u) * kThreads + tid) * kQuad;
+					G[u] = load_quad<GT, NT>(a.g, idx[u], sc);
+					M[u] = load_quad<MT, NT>(a.m, idx[u], 1.0f);
+					V[u] = load_quad<MT, NT>(a.v, idx[u], 1.0f);
+					P[u] = load_quad<kF32, NT>(a.p, idx[u], 1.0f);
+				}
+#pragma unroll
+				for (int u = 0; u < U; u++) {
+#pragma unroll
+					for (int k = 0; k < kQuad; k++) {
+						const Elem e = adam_elem(P[u][k], G[u][k], M[u][k], V[u][k],
+						    gs, a.c, decay);
+
+						P[u][k] = e.p;
+						M[u][k] = e.m;
+						V[u][k] = e.v;
+					}
+				}
+#pragma unroll
+				for (int u = 0; u < U; u++) {
+					store_quad<kF32, NT>(a.p, idx[u], P[u]);
+					store_quad<MT, NT>(a.m, idx[u], M[u]);
+					store_quad<MT, NT>(a.v, idx[u], V[u]);
+					zero_quad<GT, NT>(a.g, idx[u]);
+					if (twin)
+						store_quad<kBF16, NT>(a.twin, idx[u], P[u]);
+				}
+			}
+		} else {
+			for (int64_t i = base + tid; i < end; i += kThreads) {
+				uint32_t flags = a.uniform_flags;
+				float sc = 1.0f;
+
+				if (a.segs) {
+					while (i >= a.segs[s].end)
+						s++;
+					flags = a.segs[s].flags;
+				}
+				if (GT == kFP8)
+					sc = a.gscale[s];
+				const Elem e = adam_elem(a.p[i], load_one<GT>(a.g, i, sc),
+				    load_one<MT>(a.m, i, 1.0f), load_one<MT>(a.v, i, 1.0f), gs, a.c,
+				    a.c.decay_on && (flags & kSegDecay) != 0);
+
+				a.p[i] = e.p;
+				store_one<MT>(a.m, i, e.m);
+				store_one<MT>(a.v, i, e.v);
+				zero_one<GT>(a.g, i);
+				if ((flags & kSegTwin) != 0 && a.twin != nullptr)
+					a.twin[i] = (uint16_t)bf16_rne(e.p);
+			}
+		}
+	}
+}
+
+/* ---- helpers -------------------------------------------------------------- */
+
+/* dst[i] = bf16(src[i]), round to nearest even (seed of the twins, gpu_cuda.cu:1497-1513). */
+__global__ __launch_bounds__(kThreads) void f32_to_bf16_kernel(uint16_t *dst,
+	const float *src, int64_t n, int vec_ok)
+{
+	const int64_t n4 = vec_ok ? n / kQuad : 0;
+	const int64_t stride = (int64_t)gridDim.x * kThreads;
+
+	for (int64_t q = (int64_t)blockIdx.x * kThreads + threadIdx.x; q < n4; q += stride) {
+		const f32x4 x = *(const f32x4 *)(src + q * kQuad);
+
+		store_quad<kBF16, false>(dst, q * kQuad, x);
+	}
+	for (int64_t i = n4 * kQuad + (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n;
+	    i += stride)
+		dst[i] = (uint16_t)bf16_rne(src[i]);
+}
+
+/* Byte fill on the stream (a kernel, so it can sit in a captured graph). */
+__global__ __launch_bounds__(kThreads) void fill_bytes_kernel(uint8_t *dst, uint32_t pattern,
+	size_t nbytes, size_t head, size_t n16)
+{
+	typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+	const size_t stride = (size_t)gridDim.x * kThreads;
+	const size_t gid = (size_t)blockIdx.x * kThreads + threadIdx.x;
+	const u32x4 w = {pattern, pattern, pattern, pattern};
+
+	/* [0, head) bytes up to 16-byte alignment, n16 aligned 16-byte words, then the rest. */
+	for (size_t i = gid; i < head; i += stride)
+		dst[i] = (uint8_t)pattern;
+	for (size_t i = gid; i < n16; i += stride)
+		*(u32x4 *)(dst + head + i * 16) = w;
+	for (size_t i = head + n16 * 16 + gid; i < nbytes; i += stride)
+		dst[i] = (uint8_t)pattern;
+}
+
+/* ---- host side ------------------------------------------------------------ */
+
+static int env_int(const char *name, int dflt, int lo, int hi)
+{
+	const char *e = getenv(name);
+	int v;
+
+	if (!e || !*e)
+		return dflt;
+	v = atoi(e);
+	if (v < lo)
+		v = lo;
+	if (v > hi)
+		v = hi;
+	return v;
+}
+
+static int cu_count(void)
+{
+	static int cus;
+
+	if (!cus) {
+		int dev = 0;
+		int n = 0;
+
+		if (hipGetDevice(&dev) != hipSuccess
+		    || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev)
+		    != hipSuccess || n <= 0)
+			n = 256;
+		cus = n;
+	}
+	return cus;
+}
+
+/* ANNI_BLOCKS_PER_CU: persistent workgroups per compute unit (default 8). */
+int grid_for(int64_t n)
+{
+	static int per_cu;
+	int64_t tiles = (n + kTile - 1) / kTile;
+	int64_t g;
+
+	if (!per_cu)
+		per_cu = env_int("ANNI_BLOCKS_PER_CU", 8, 1, 32);
+	g = (int64_t)cu_count() * per_cu;
+	if (g > kMaxPartials)
+		g = kMaxPartials;
+	if (g > tiles)
+		g = tiles;
+	if (g < 1)
+		g = 1;
+	return (int)g;
+}
+
+/* ANNI_NT=0 switches the streaming (non-temporal) cache hint off. */
+static bool nt_on(void)
+{
+	static int on = -1;
+
+	if (on < 0)
+		on = env_int("ANNI_NT", 1, 0, 1);
+	return on != 0;
+}
+
+static bool aligned(const void *p, uintptr_t a)
+{
+	return ((uintptr_t)p & (a - 1)) == 0;
+}
+
+static uintptr_t quad_bytes(int type)
+{
+	return type == kF32 ? 16 : type == kBF16 ? 8 : 4;
+}
+
+static int check_flat(const Flat &f, bool need_state)
+{
+	if (!f.g || f.n <= 0)
+		return -1;
+	if (f.grad_type < kF32 || f.grad_type > kFP8)
+		return -1;
+	if (f.grad_type == kFP8 && !f.gscale)
+		return -1;
+	if ((f.segs == nullptr) != (f.tile_seg == nullptr))
+		return -1;
+	if (need_state) {
+		if (!f.p || !f.m || !f.v)
+			return -1;
+		if (f.moment_type != kF32 && f.moment_type != kBF16)
+			return -1;
+	}
+	return 0;
+}
+
+int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *partials,
+	int *n_partials)
+{
+	SumsqArgs a;
+	int grid;
+
+	if (check_flat(f, false) != 0 || !partials || !n_partials)
+		return -1;
+	grid = grid_for(f.n);
+	a.g = f.g;
+	a.n = f.n;
+	a.segs = f.segs;
+	a.tile_seg = f.tile_seg;
+	a.gscale = f.gscale;
+	a.grad_scale = grad_scale;
+	a.partials = partials;
+	a.vec_ok = aligned(f.g, quad_bytes(f.grad_type)) ? 1 : 0;
+#define SUMSQ_LAUNCH(GT) \
+	do { \
+		if (nt_on()) \
+			hipLaunchKernelGGL((sumsq_kernel<GT, true>), dim3(grid), dim3(kThreads), 0, st, a); \
+		else \
+			hipLaunchKernelGGL((sumsq_kernel<GT, false>), dim3(grid), dim3(kThreads), 0, st, a); \
+	} while (0)
+	if (f.grad_type == kF32)
+		SUMSQ_LAUNCH(kF32);
+	else if (f.grad_type == kBF16)
+		SUMSQ_LAUNCH(kBF16);
+	else
+		SUMSQ_LAUNCH(kFP8);
+#undef SUMSQ_LAUNCH
+	*n_partials = grid;
+	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int launch_finalize(hipStream_t st, const double *partials, int n_partials, double clip,
+	int skip_nonfinite, double grad_scale, StepState *state)
+{
+	FinalizeArgs a;
+
+	if (!partials || n_partials <= 0 || !state)
+		return -1;
+	a.partials = partials;
+	a.n_partials = n_partials;
+	a.clip = clip;
+	a.skip_nonfinite = skip_nonfinite;
+	a.grad_scale = grad_scale;
+	a.state = state;
+	hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kThreads), 0, st, a);
+	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+#ifndef ANNI_UPDATE_UNROLL
+#define ANNI_UPDATE_UNROLL 2
+#endif
+
+template <int GT, int MT>
+static void update_launch(hipStream_t st, int grid, const UpdateArgs &a)
+{
+	if (nt_on())
+		hipLaunchKernelGGL((adam_update_kernel<GT, MT, ANNI_UPDATE_UNROLL, true>),
+		    dim3(grid), dim3(kThreads), 0, st, a);
+	else
+		hipLaunchKernelGGL((adam_update_kernel<GT, MT, ANNI_UPDATE_UNROLL, false>),
+		    dim3(grid), dim3(kThreads), 0, st, a);
+}
+
+int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double grad_scale,
+	const NormIn &norm)
+{
+	UpdateArgs a;
+	int grid;
+
+	if (check_flat(f, true) != 0)
+		return -1;
+	if (norm.use_norm && (!norm.partials || norm.n_partials <= 0))
+		return -1;
+	grid = grid_for(f.n);
+	a.p = f.p;
+	a.g = f.g;
+	a.m = f.m;
+	a.v = f.v;
+	a.twin = f.twin;
+	a.n = f.n;
+	a.segs = f.segs;
+	a.tile_seg = f.tile_seg;
+	a.gscale = f.gscale;
+	a.uniform_flags = f.uniform_flags;
+	a.vec_ok = aligned(f.p, 16) && aligned(f.g, quad_bytes(f.grad_type))
+	    && aligned(f.m, quad_bytes(f.moment_type)) && aligned(f.v, quad_bytes(f.moment_type))
+	    && (!f.twin || aligned(f.twin, 8)) ? 1 : 0;
+	a.c = c;
+	a.grad_scale = grad_scale;
+	a.use_norm = norm.use_norm;
+	a.skip_nonfinite = norm.skip_nonfinite;
+	a.partials = norm.partials;
+	a.n_partials = norm.n_partials;
+	a.clip = norm.clip;
+	a.state = norm.state;
+	if (f.moment_type == kF32) {
+		if (f.grad_type == kF32)
+			update_launch<kF32, kF32>(st, grid, a);
+		else if (f.grad_type == kBF16)
+			update_launch<kBF16, kF32>(st, grid, a);
+		else
+			update_launch<kFP8, kF32>(st, grid, a);
+	} else {
+		if (f.grad_type == kF32)
+			update_launch<kF32, kBF16>(st, grid, a);
+		else if (f.grad_type == kBF16)
+			update_launch<kBF16, kBF16>(st, grid, a);
+		else
+			update_launch<kFP8, kBF16>(st, grid, a);
+	}
+	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+static int helper_grid(int64_t work_items)
+{
+	int64_t g = (work_items + kThreads - 1) / kThreads;
+	int64_t cap = (int64_t)cu_count() * 8;
+
+	if (g > cap)
+		g = cap;
+	if (g < 1)
+		g = 1;
+	return (int)g;
+}
+
+int launch_f32_to_bf16(hipStream_t st, uint16_t *dst, const float *src, int64_t n)
+{
+	if (!dst || !src || n <= 0)
+		return -1;
+	hipLaunchKernelGGL(f32_to_bf16_kernel, dim3(helper_grid(n / kQuad + 1)), dim3(kThreads),
+	    0, st, dst, src, n, aligned(src, 16) && aligned(dst, 8) ? 1 : 0);
+	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int launch_fill_bytes(hipStream_t st, void *dst, int value, size_t nbytes)
+{
+	const uint32_t b = (uint32_t)(value & 0xff);
+	const uint32_t pattern = b | (b << 8) | (b << 16) | (b << 24);
+	size_t head;
+	size_t n16;
+
+	if (!dst || nbytes == 0)
+		return -1;
+	head = (16 - ((uintptr_t)dst & 15)) & 15;
+	if (head > nbytes)
+		head = nbytes;
+	n16 = (nbytes - head) / 16;
+	hipLaunchKernelGGL(fill_bytes_kernel, dim3(helper_grid((int64_t)n16 + 16)), dim3(kThreads),
+	    0, st, (uint8_t *)dst, pattern, nbytes, head, n16);
+	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+} /* namespace anni */

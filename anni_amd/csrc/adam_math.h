@@ -1,0 +1,118 @@
+/*
+** Per-element arithmetic of the AdamW step, shared by every kernel variant.
+**
+** The parity target is the reference's HOST loop (lang/lm_adam.c:587-598), which
+** computes in double and stores float after each of m, v, the Adam step on p and
+** the decay on p.  The device code below performs the same IEEE-754 double
+** operations in the same order (this library is compiled with -ffp-contract=off,
+** so no multiply-add is fused), which makes p, m and v bit-identical to the host
+** loop whenever the effective gradient scale is the same double.
+*/
+#ifndef ANNI_ADAM_MATH_H__
+#define ANNI_ADAM_MATH_H__
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace anni {
+
+/* Scalars of one step, computed on the host in double as lm_adam.c:571-572 does. */
+struct StepConsts {
+	double	beta1;
+	double	omb1;	/* 1.0 - beta1 */
+	double	beta2;
+	double	omb2;	/* 1.0 - beta2 */
+	double	eps;
+	double	bc1;	/* 1 - beta1^t */
+	double	bc2;	/* 1 - beta2^t */
+	double	lr;
+	double	lr_wd;	/* lr * weight_decay (lm_adam.c:595 multiplies these first) */
+	int	decay_on;	/* weight_decay > 0 (lm_adam.c:594); per-tensor flags select where */
+};
+
+/* New p, m, v of one element. */
+struct Elem {
+	float	p;
+	float	m;
+	float	v;
+};
+
+/*
+** g is the gradient element as a float; gs the effective gradient scale.
+** Rounding points: m, v (float), p after the step, p after the decay.
+*/
+__device__ __forceinline__ Elem adam_elem(float p, float g, float m, float v, double gs,
+	const StepConsts &c, bool decay)
+{
+	Elem r;
+	const double x = (double)g * gs;
+
+	r.m = (float)(c.beta1 * (double)m + c.omb1 * x);
+	r.v = (float)(c.beta2 * (double)v + (c.omb2 * x) * x);
+	const double mhat = (double)r.m / c.bc1;
+	const double vhat = (double)r.v / c.bc2;
+	r.p = (float)((double)p - (c.lr * mhat) / (sqrt(vhat) + c.eps));
+	if (decay)
+		r.p = (float)((double)r.p - c.lr_wd * (double)r.p);
+	return r;
+}
+
+/* float -> bfloat16 bits, round to nearest even; NaN stays NaN (quiet bit set). */
+__device__ __forceinline__ uint32_t bf16_rne(float x)
+{
+	uint32_t u = __float_as_uint(x);
+
+	if ((u & 0x7fffffffu) > 0x7f800000u)
+		return (u >> 16) | 0x0040u;
+	u += 0x7fffu + ((u >> 16) & 1u);
+	return u >> 16;
+}
+
+__device__ __forceinline__ float bf16_widen(uint32_t h)
+{
+	return __uint_as_float(h << 16);
+}
+
+/* OCP E4M3 byte -> float (exact): bias 7, subnormals f/8 * 2^-6, S.1111.111 = NaN, no infinities. */
+__device__ __forceinline__ float fp8_e4m3_decode(uint32_t q)
+{
+	const uint32_t s = (q & 0x80u) << 24;
+	const uint32_t e = (q >> 3) & 15u;
+	const uint32_t f = q & 7u;
+	uint32_t bits;
+
+	if (e == 0u)
+		bits = __float_as_uint((float)f * 0x1p-9f);
+	else if (e == 15u && f == 7u)
+		bits = 0x7fc00000u;
+	else
+		bits = ((e + 120u) << 23) | (f << 20);
+	return __uint_as_float(s | bits);
+}
+
+/* float -> OCP E4M3 byte: round to nearest even, saturate to +-448, NaN -> S.1111.111. */
+__device__ __forceinline__ uint32_t fp8_e4m3_encode(float x)
+{
+	const uint32_t u = __float_as_uint(x);
+	const uint32_t s = (u >> 24) & 0x80u;
+	const float a = __uint_as_float(u & 0x7fffffffu);
+	int e;
+	int q;
+
+	if (a != a)
+		return s | 0x7fu;
+	if (a >= 448.0f)
+		return s | 0x7eu;
+	if (a < 0.015625f)
+		return s | (uint32_t)(int)rintf(a * 512.0f);	/* subnormal grid, step 2^-9 */
+	e = (int)((u >> 23) & 0xffu) - 127;			/* a = 1.xxx * 2^e, e in [-6, 8] */
+	q = (int)rintf(ldexpf(a, 3 - e));			/* 8..16 */
+	if (q == 16) {
+		q = 8;
+		e += 1;
+	}
+	return s | (uint32_t)((e + 7) << 3) | (uint32_t)(q - 8);
+}
+
+} /* namespace anni */
+#endif

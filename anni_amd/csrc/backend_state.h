@@ -1,0 +1,22 @@
+/*
+** State shared by the C-ABI translation units of libanni_gpu_hip.so: the one
+** in-order compute stream every operation is issued on (the reference's g_st,
+** num/gpu_cuda.cu:36-44) and a couple of helpers.
+*/
+#ifndef ANNI_BACKEND_STATE_H__
+#define ANNI_BACKEND_STATE_H__
+
+#include <hip/hip_runtime.h>
+
+namespace anni {
+
+/* True once a device is present and the compute stream exists. */
+bool		device_ready(void);
+hipStream_t	compute_stream(void);
+/* NULL restores the library's own stream. */
+void		set_compute_stream(hipStream_t st);
+/* Remembers the first HIP error for gpu_debug_last_error; returns err == hipSuccess. */
+bool		hip_ok(hipError_t err, const char *what);
+
+} /* namespace anni */
+#endif

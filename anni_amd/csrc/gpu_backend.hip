@@ -1,0 +1,500 @@
+/*
+** libanni_gpu_hip.so -- the optimizer-step subset of AnnI's backend C ABI
+** (num/gpu.h) on MI355X.  See include/anni_gpu.h for the contract of each entry
+** point and the reference line it stands in for.
+*/
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <mutex>
+#include "adam_kernels.h"
+#include "anni_gpu.h"
+#include "backend_state.h"
+
+namespace anni {
+
+static std::once_flag g_init_once;
+static bool g_ready;
+static hipStream_t g_own_stream;
+static hipStream_t g_stream;
+static std::mutex g_mu;			/* guards everything below */
+static char g_err[256];
+
+static void init_once(void)
+{
+	int n = 0;
+	const char *off = getenv("ANNI_GPU_DISABLE");
+
+	if (off && off[0] == '1')
+		return;
+	if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+		(void)hipGetLastError();
+		return;
+	}
+	/* A blocking stream: synchronous hipMemcpy calls order themselves with it. */
+	if (hipStreamCreate(&g_own_stream) != hipSuccess) {
+		(void)hipGetLastError();
+		return;
+	}
+	g_stream = g_own_stream;
+	g_ready = true;
+}
+
+bool device_ready(void)
+{
+	std::call_once(g_init_once, init_once);
+	return g_ready;
+}
+
+hipStream_t compute_stream(void)
+{
+	return g_stream;
+}
+
+void set_compute_stream(hipStream_t st)
+{
+	g_stream = st ? st : g_own_stream;
+}
+
+bool hip_ok(hipError_t err, const char *what)
+{
+	if (err == hipSuccess)
+		return true;
+	std::lock_guard<std::mutex> lk(g_mu);
+	if (!g_err[0])
+		snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(err));
+	return false;
+}
+
+/* ---- state of the flat drop-in path ------------------------------------- */
+
+static int g_prec = GPU_PREC_FP32;
+static double g_wd;
+static unsigned g_epoch;
+static void *g_twin_bf16;		/* borrowed registration (gpu_adam_set_bf16_flat) */
+static const float *g_twin_fp32;
+static int g_twin_n;
+
+#define PIN_SLOTS 256			/* as the reference's table, gpu_cuda.cu:2980 */
+static const void *g_pinned[PIN_SLOTS];
+static int g_pinned_n;
+
+/* Scratch of the flat path: sum-of-squares partials + the step state, and a pinned result word. */
+static double *g_partials;
+static StepState *g_state;
+static double *g_host_result;
+
+static bool scratch_ready(void)
+{
+	std::lock_guard<std::mutex> lk(g_mu);
+
+	if (g_partials)
+		return true;
+	void *d = nullptr;
+	void *h = nullptr;
+
+	if (hipMalloc(&d, sizeof(double) * kMaxPartials + sizeof(StepState)) != hipSuccess
+	    || hipHostMalloc(&h, sizeof(StepState), hipHostMallocDefault) != hipSuccess) {
+		(void)hipGetLastError();
+		if (d)
+			(void)hipFree(d);
+		return false;
+	}
+	g_partials = (double *)d;
+	g_state = (StepState *)(g_partials + kMaxPartials);
+	g_host_result = (double *)h;
+	return true;
+}
+
+/* ---- ANN_OP_PROF=1: event pairs around the step's launches ---------------- */
+
+struct ProfSlot {
+	hipEvent_t	a;
+	hipEvent_t	b;
+	int		kind;	/* 0 sumsq, 1 update */
+};
+#define PROF_SLOTS 64
+static ProfSlot g_prof[PROF_SLOTS];
+static int g_prof_n;
+static double g_prof_ms[2];
+static int g_prof_calls[2];
+
+static bool prof_on(void)
+{
+	static int on = -1;
+
+	if (on < 0) {
+		const char *e = getenv("ANN_OP_PROF");
+
+		on = (e && e[0] == '1') ? 1 : 0;
+	}
+	return on == 1;
+}
+
+static void prof_resolve(void)
+{
+	for (int i = 0; i < g_prof_n; i++) {
+		float ms = 0.0f;
+
+		if (hipEventSynchronize(g_prof[i].b) == hipSuccess
+		    && hipEventElapsedTime(&ms, g_prof[i].a, g_prof[i].b) == hipSuccess) {
+			g_prof_ms[g_prof[i].kind] += ms;
+			g_prof_calls[g_prof[i].kind]++;
+		}
+		(void)hipEventDestroy(g_prof[i].a);
+		(void)hipEventDestroy(g_prof[i].b);
+	}
+	g_prof_n = 0;
+}
+
+struct ProfScope {
+	int	slot;
+
+	explicit ProfScope(int kind) : slot(-1)
+	{
+		if (!prof_on())
+			return;
+		if (g_prof_n == PROF_SLOTS)
+			prof_resolve();
+		ProfSlot &s = g_prof[g_prof_n];
+
+		if (hipEventCreate(&s.a) != hipSuccess)
+			return;
+		if (hipEventCreate(&s.b) != hipSuccess) {
+			(void)hipEventDestroy(s.a);
+			return;
+		}
+		s.kind = kind;
+		(void)hipEventRecord(s.a, g_stream);
+		slot = g_prof_n++;
+	}
+	~ProfScope()
+	{
+		if (slot >= 0)
+			(void)hipEventRecord(g_prof[slot].b, g_stream);
+	}
+};
+
+} /* namespace anni */
+
+using namespace anni;
+
+extern "C" {
+
+int gpu_available(void)
+{
+	return device_ready() ? 1 : 0;
+}
+
+const char *gpu_backend_name(void)
+{
+	return "hip-gfx950";
+}
+
+int gpu_mem_info(size_t *free_bytes, size_t *total_bytes)
+{
+	size_t f = 0;
+	size_t t = 0;
+
+	if (!device_ready() || !hip_ok(hipMemGetInfo(&f, &t), "hipMemGetInfo"))
+		return -1;
+	if (free_bytes)
+		*free_bytes = f;
+	if (total_bytes)
+		*total_bytes = t;
+	return 0;
+}
+
+void gpu_device_sync(void)
+{
+	hipError_t err;
+
+	if (!device_ready())
+		return;
+	err = hipDeviceSynchronize();
+	if (err != hipSuccess) {
+		fprintf(stderr, "gpu_device_sync: %s\n", hipGetErrorString(err));
+		(void)hip_ok(err, "hipDeviceSynchronize");
+	} else if (prof_on()) {
+		std::lock_guard<std::mutex> lk(g_mu);
+		prof_resolve();
+	}
+}
+
+int gpu_stream_sync(void)
+{
+	if (!device_ready())
+		return -1;
+	return hip_ok(hipStreamSynchronize(g_stream), "hipStreamSynchronize") ? 0 : -1;
+}
+
+void gpu_set_compute_prec(int prec)
+{
+	g_prec = prec == GPU_PREC_BF16 ? GPU_PREC_BF16 : GPU_PREC_FP32;
+}
+
+const char *gpu_debug_last_error(void)
+{
+	static thread_local char out[256];
+	std::lock_guard<std::mutex> lk(g_mu);
+
+	if (!g_err[0] && device_ready()) {
+		hipError_t err = hipGetLastError();
+
+		if (err != hipSuccess)
+			snprintf(g_err, sizeof(g_err), "%s", hipGetErrorString(err));
+	}
+	memcpy(out, g_err, sizeof(out));
+	g_err[0] = '\0';
+	return out;
+}
+
+void gpu_op_prof_dump(void)
+{
+	static const char *name[2] = { "grad_sumsq", "adam_step" };
+
+	if (!prof_on() || !device_ready())
+		return;
+	std::lock_guard<std::mutex> lk(g_mu);
+	prof_resolve();
+	for (int k = 0; k < 2; k++) {
+		if (!g_prof_calls[k])
+			continue;
+		fprintf(stderr, "[op-prof] %-12s %8.3f ms  %d calls\n", name[k], g_prof_ms[k],
+		    g_prof_calls[k]);
+		g_prof_ms[k] = 0.0;
+		g_prof_calls[k] = 0;
+	}
+}
+
+/* ---- memory --------------------------------------------------------------- */
+
+void *gpu_malloc(size_t nbytes)
+{
+	void *p = nullptr;
+
+	if (nbytes == 0 || !device_ready())
+		return nullptr;
+	if (!hip_ok(hipMalloc(&p, nbytes), "hipMalloc")) {
+		(void)hipGetLastError();
+		return nullptr;
+	}
+	return p;
+}
+
+void gpu_free(void *p)
+{
+	if (!p || !device_ready())
+		return;
+	{
+		std::lock_guard<std::mutex> lk(g_mu);
+
+		/* A freed flat must not stay registered: the address may be reused. */
+		if (p == g_twin_bf16 || p == (const void *)g_twin_fp32) {
+			g_twin_bf16 = nullptr;
+			g_twin_fp32 = nullptr;
+			g_twin_n = 0;
+		}
+	}
+	(void)hip_ok(hipFree(p), "hipFree");
+}
+
+int gpu_memcpy_h2d(void *dst, const void *src, size_t nbytes)
+{
+	if (!dst || !src || nbytes == 0 || !device_ready())
+		return -1;
+	return hip_ok(hipMemcpyAsync(dst, src, nbytes, hipMemcpyHostToDevice, g_stream),
+	    "h2d") ? 0 : -1;
+}
+
+int gpu_memcpy_d2h(void *dst, const void *src, size_t nbytes)
+{
+	if (!dst || !src || nbytes == 0 || !device_ready())
+		return -1;
+	if (!hip_ok(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, g_stream), "d2h"))
+		return -1;
+	return hip_ok(hipStreamSynchronize(g_stream), "d2h sync") ? 0 : -1;
+}
+
+/*
+** The reference page-locks the caller's range here (gpu_cuda.cu:2982-3001).
+** This backend only remembers it: an asynchronous copy into pageable memory is
+** staged by the runtime and has landed by the next gpu_stream_sync, which is
+** all lang/lm_adam.c:407-413,500 relies on.
+*/
+int gpu_host_pin(void *p, size_t nbytes)
+{
+	if (!p || nbytes == 0 || !device_ready())
+		return -1;
+	std::lock_guard<std::mutex> lk(g_mu);
+
+	for (int i = 0; i < g_pinned_n; i++)
+		if (g_pinned[i] == p)
+			return 0;
+	if (g_pinned_n >= PIN_SLOTS)
+		return -1;
+	g_pinned[g_pinned_n++] = p;
+	return 0;
+}
+
+void gpu_host_forget(const void *host)
+{
+	std::lock_guard<std::mutex> lk(g_mu);
+
+	for (int i = 0; i < g_pinned_n; i++)
+		if (g_pinned[i] == host) {
+			g_pinned[i] = g_pinned[--g_pinned_n];
+			return;
+		}
+}
+
+int gpu_memcpy_d2h_async(void *dst, const void *src, size_t nbytes)
+{
+	if (!dst || !src || nbytes == 0 || !device_ready())
+		return -1;
+	return hip_ok(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, g_stream),
+	    "d2h async") ? 0 : -1;
+}
+
+int gpu_memcpy_d2d(void *dst, const void *src, size_t nbytes)
+{
+	if (!dst || !src || nbytes == 0 || !device_ready())
+		return -1;
+	return hip_ok(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToDevice, g_stream),
+	    "d2d") ? 0 : -1;
+}
+
+int gpu_memset(void *dst, int value, size_t nbytes)
+{
+	if (!dst || nbytes == 0 || !device_ready())
+		return -1;
+	return launch_fill_bytes(g_stream, dst, value, nbytes);
+}
+
+void *gpu_host_alloc(size_t nbytes)
+{
+	void *p = nullptr;
+
+	if (nbytes == 0 || !device_ready())
+		return nullptr;
+	if (!hip_ok(hipHostMalloc(&p, nbytes, hipHostMallocDefault), "hipHostMalloc")) {
+		(void)hipGetLastError();
+		return nullptr;
+	}
+	return p;
+}
+
+void gpu_host_free(void *p)
+{
+	if (p && device_ready())
+		(void)hip_ok(hipHostFree(p), "hipHostFree");
+}
+
+/* ---- BF16 twins ------------------------------------------------------------- */
+
+void gpu_adam_set_bf16_flat(void *bf16, const ann_real *fp32, int n)
+{
+	std::lock_guard<std::mutex> lk(g_mu);
+
+	g_twin_bf16 = bf16;
+	g_twin_fp32 = fp32;
+	g_twin_n = (bf16 && fp32 && n > 0) ? n : 0;
+}
+
+int gpu_adam_seed_bf16_flat(void *bf16, const ann_real *fp32, int n)
+{
+	if (!bf16 || !fp32 || n <= 0 || !device_ready())
+		return -1;
+	return launch_f32_to_bf16(g_stream, (uint16_t *)bf16, fp32, n);
+}
+
+void gpu_half_wt_invalidate(const ann_real *fp32_dev)
+{
+	(void)fp32_dev;		/* no per-matrix twin cache here: the flat twin is always current */
+	std::lock_guard<std::mutex> lk(g_mu);
+	g_epoch++;
+}
+
+unsigned gpu_param_epoch(void)
+{
+	std::lock_guard<std::mutex> lk(g_mu);
+	return g_epoch;
+}
+
+/* ---- the optimizer step -------------------------------------------------------- */
+
+void gpu_adam_set_weight_decay(double wd)
+{
+	g_wd = wd > 0.0 ? wd : 0.0;
+}
+
+int gpu_grad_sumsq(const ann_real *d_x, int n, double *out)
+{
+	Flat f;
+	int np = 0;
+
+	if (!d_x || n <= 0 || !out || !device_ready() || !scratch_ready())
+		return -1;
+	memset(&f, 0, sizeof(f));
+	f.g = (void *)d_x;
+	f.n = n;
+	f.grad_type = kF32;
+	{
+		ProfScope prof(0);
+
+		if (launch_sumsq(g_stream, f, 1.0, g_partials, &np) != 0
+		    || launch_finalize(g_stream, g_partials, np, 0.0, 0, 1.0, g_state) != 0)
+			return -1;
+	}
+	if (!hip_ok(hipMemcpyAsync(g_host_result, &g_state->sumsq, sizeof(double),
+	    hipMemcpyDeviceToHost, g_stream), "sumsq d2h")
+	    || !hip_ok(hipStreamSynchronize(g_stream), "sumsq sync"))
+		return -1;
+	*out = *g_host_result;
+	return 0;
+}
+
+int gpu_adam_step_dev_bf16(ann_real *d_param, void *d_param_bf16, ann_real *d_grad,
+	ann_real *d_m, ann_real *d_v, int n, double lr, double beta1, double beta2, double eps,
+	int t, double grad_scale)
+{
+	Flat f;
+	StepConsts c;
+	NormIn norm;
+
+	if (!d_param || !d_grad || !d_m || !d_v || n <= 0 || lr <= 0.0 || t < 1)
+		return -1;
+	if (!device_ready())
+		return -1;
+	c.bc1 = 1.0 - pow(beta1, (double)t);		/* lm_adam.c:571-572 */
+	c.bc2 = 1.0 - pow(beta2, (double)t);
+	if (c.bc1 <= 0.0 || c.bc2 <= 0.0)
+		return -1;
+	c.beta1 = beta1;
+	c.omb1 = 1.0 - beta1;
+	c.beta2 = beta2;
+	c.omb2 = 1.0 - beta2;
+	c.eps = eps;
+	c.lr = lr;
+	c.decay_on = g_wd > 0.0 ? 1 : 0;
+	c.lr_wd = lr * g_wd;
+	memset(&f, 0, sizeof(f));
+	f.p = d_param;
+	f.g = d_grad;
+	f.m = d_m;
+	f.v = d_v;
+	f.twin = (d_param_bf16 && g_prec == GPU_PREC_BF16) ? (uint16_t *)d_param_bf16 : nullptr;
+	f.n = n;
+	f.grad_type = kF32;
+	f.moment_type = kF32;
+	f.uniform_flags = (g_wd > 0.0 ? kSegDecay : 0u) | (f.twin ? kSegTwin : 0u);
+	memset(&norm, 0, sizeof(norm));
+	ProfScope prof(1);
+
+	return launch_update(g_stream, f, c, grad_scale, norm);
+}
+
+} /* extern "C" */

@@ -1,0 +1,160 @@
+"""Host-side mirror of the reference's lm_adam interface over the device arena.
+
+Names and argument meaning follow lang/lm_adam.h:56-78 (create, step,
+step_scaled, zero_grad, free) and lang/lm_train.c:98-124 (step_lr); the work is
+done by libanni_gpu_hip.so through its C ABI (include/anni_adam.h).  numpy is
+used only to move test data; nothing here computes the update.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import lib as _l
+
+_NP = {_l.F32: np.float32, _l.BF16: np.uint16, _l.FP8_E4M3: np.uint8}
+
+
+def step_lr(base_lr, step, warmup=0, decay_steps=0, kind="none", sched_from=0):
+    """lm_train_step_lr with its setters applied first (lang/lm_train.c:98-124,398-411)."""
+    L = _l.load()
+    L.anni_lr_set_schedule(warmup, decay_steps, kind.encode())
+    L.anni_lr_set_sched_from(sched_from)
+    return L.anni_lr_step(base_lr, step)
+
+
+class DeviceBuffer:
+    """A gpu_malloc'ed range (freed with gpu_free)."""
+
+    def __init__(self, nbytes):
+        self.L = _l.require_gpu()
+        self.nbytes = int(nbytes)
+        self.ptr = self.L.gpu_malloc(self.nbytes)
+        if not self.ptr:
+            raise MemoryError("gpu_malloc(%d)" % self.nbytes)
+
+    def upload(self, arr, offset=0):
+        arr = np.ascontiguousarray(arr)
+        assert offset + arr.nbytes <= self.nbytes
+        if arr.nbytes and self.L.gpu_memcpy_h2d(self.ptr + offset, arr.ctypes.data,
+                                                arr.nbytes) != 0:
+            raise RuntimeError("gpu_memcpy_h2d failed")
+        if self.L.gpu_stream_sync() != 0:
+            raise RuntimeError("gpu_stream_sync failed")
+
+    def download(self, dtype, count, offset=0):
+        out = np.empty(count, dtype=dtype)
+        assert offset + out.nbytes <= self.nbytes
+        if out.nbytes and self.L.gpu_memcpy_d2h(out.ctypes.data, self.ptr + offset,
+                                                out.nbytes) != 0:
+            raise RuntimeError("gpu_memcpy_d2h failed")
+        return out
+
+    def free(self):
+        if self.ptr:
+            self.L.gpu_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class LmAdam:
+    """lm_adam over a list of tensors ((n, flags) pairs or (name, n, flags) triples)."""
+
+    def __init__(self, tensors, grad_type=_l.F32, moment_type=_l.F32, twins=True,
+                 skip_nonfinite=False, own_grad=True, beta1=0.9, beta2=0.999, eps=1e-8,
+                 weight_decay=0.0, grad_clip=0.0):
+        self.L = _l.require_gpu()
+        rows = [(t[-2], t[-1]) for t in tensors]
+        self.names = [t[0] if len(t) == 3 else "t%d" % i for i, t in enumerate(tensors)]
+        arr = (_l.Tensor * len(rows))(*[_l.Tensor(int(n), int(f)) for n, f in rows])
+        cfg = _l.Config(grad_type, moment_type, int(twins), int(skip_nonfinite), int(own_grad))
+        self.h = self.L.anni_adam_create(arr, len(rows), C.byref(cfg))
+        if not self.h:
+            raise RuntimeError("anni_adam_create failed: %s"
+                               % self.L.gpu_debug_last_error().decode())
+        self.grad_type, self.moment_type = grad_type, moment_type
+        o = self.h.contents
+        o.beta1, o.beta2, o.eps = beta1, beta2, eps
+        o.weight_decay, o.grad_clip = weight_decay, grad_clip
+        self.sizes = [n for n, _f in rows]
+        self.offsets = [self.L.anni_adam_tensor_offset(self.h, i) for i in range(len(rows))]
+
+    # -- the reference's public fields ------------------------------------------------
+    @property
+    def o(self):
+        return self.h.contents
+
+    @property
+    def n(self):
+        return self.o.n
+
+    @property
+    def t(self):
+        return self.o.t
+
+    # -- the reference's functions ------------------------------------------------------
+    def step_scaled(self, lr, grad_scale=1.0):
+        rc = self.L.anni_adam_step_scaled(self.h, lr, grad_scale)
+        if rc < 0:
+            raise RuntimeError("anni_adam_step_scaled failed: %s"
+                               % self.L.gpu_debug_last_error().decode())
+        return rc
+
+    def step(self, lr):
+        return self.step_scaled(lr, 1.0)
+
+    def zero_grad(self):
+        if self.L.anni_adam_zero_grad(self.h) != 0:
+            raise RuntimeError("anni_adam_zero_grad failed")
+
+    def seed_twins(self):
+        if self.L.anni_adam_seed_twins(self.h) != 0:
+            raise RuntimeError("anni_adam_seed_twins failed")
+
+    def sync_stats(self):
+        if self.L.anni_adam_sync_stats(self.h) != 0:
+            raise RuntimeError("anni_adam_sync_stats failed")
+        return self.o
+
+    def bind_grad(self, ptr):
+        if self.L.anni_adam_bind_grad(self.h, ptr) != 0:
+            raise RuntimeError("anni_adam_bind_grad failed")
+
+    def free(self):
+        if getattr(self, "h", None):
+            hp = C.POINTER(_l.Adam)(self.h.contents)
+            self.L.anni_adam_free(C.byref(hp))
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+    # -- test / bench data movement --------------------------------------------------------
+    def _flat(self, which):
+        o = self.o
+        return {"param": (o.d_param, np.float32), "grad": (o.d_grad, _NP[self.grad_type]),
+                "m": (o.d_m, _NP[self.moment_type]), "v": (o.d_v, _NP[self.moment_type]),
+                "twin": (o.d_param_bf16, np.uint16), "gscale": (o.d_gscale, np.float32)}[which]
+
+    def upload(self, which, arr, offset=0):
+        ptr, dt = self._flat(which)
+        arr = np.ascontiguousarray(arr, dtype=dt)
+        if self.L.gpu_memcpy_h2d(ptr + offset * arr.itemsize, arr.ctypes.data, arr.nbytes) != 0 \
+                or self.L.gpu_stream_sync() != 0:
+            raise RuntimeError("upload(%s) failed" % which)
+
+    def download(self, which, count=None, offset=0):
+        ptr, dt = self._flat(which)
+        if count is None:
+            count = self.o.n_tensors if which == "gscale" else self.n
+        out = np.empty(count, dtype=dt)
+        if self.L.gpu_memcpy_d2h(out.ctypes.data, ptr + offset * out.itemsize, out.nbytes) != 0:
+            raise RuntimeError("download(%s) failed" % which)
+        return out

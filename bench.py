@@ -1,0 +1,259 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused AdamW + clip + bf16-twin optimizer step on one MI355X.
+
+A "step" is one pass of the optimizer over the whole parameter set of the named workload:
+the global sum of squares of the gradients (clip norm) and the fused update.  Inputs are
+synthetic and already resident in HBM when the timed region starts: parameters ~N(0, 0.02),
+zero moments, and one fresh gradient flat ~N(0, 1e-3) per step (a ring of steps+warmup flats,
+generated on the device), scaled so that about half the steps clip.  The learning rate follows
+a 100-step warmup + cosine schedule.
+
+Prints ONE JSON line.  `value` is whole-step algorithmic HBM throughput (bytes the step must
+move per parameter x parameters / step time); `roofline` is the update kernel alone, timed
+with HIP events on the library's compute stream; `cpu_baseline` is the same step on the host
+cores of this box (multithreaded restatement of the reference's loop) on a bounded sample.
+"""
+import argparse
+import ctypes as C
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+# name: (size, grad_type, moment_type, bytes/param of the norm pass, bytes/param of the update)
+WORKLOADS = {
+    "185m": ("185m", 0, 0, 4, 34),          # BASELINE config 2
+    "555m": ("555m", 0, 0, 4, 34),          # BASELINE config 3 (headline)
+    "555m-bf16": ("555m", 1, 1, 2, 22),     # BASELINE config 4
+    "1p4b-fp8": ("1p4b", 2, 0, 1, 28),      # BASELINE config 5
+}
+ELEM = {0: 4, 1: 2, 2: 1}
+STORAGE = {"185m": "f32 p/g/m/v + bf16 twin", "555m": "f32 p/g/m/v + bf16 twin",
+           "555m-bf16": "f32 p, bf16 g/m/v + bf16 twin",
+           "1p4b-fp8": "f32 p/m/v, fp8-e4m3 g with per-tensor scale + bf16 twin"}
+
+
+def make_grad_ring(L, opt, tensors, count, grad_type, seed):
+    """count gradient flats on the device, each ~N(0, 1e-3) in the workload's storage type."""
+    from anni_amd.lm_adam import DeviceBuffer
+    n = opt.n
+    ring, scales = [], []
+    stage = DeviceBuffer(n * 4) if grad_type != 0 else None
+    for k in range(count):
+        buf = DeviceBuffer(n * ELEM[grad_type])
+        dst = buf.ptr if grad_type == 0 else stage.ptr
+        assert L.anni_fill_normal_f32(dst, n, seed, 1000 + k, 0.0, 1e-3) == 0
+        sc = None
+        if grad_type == 1:
+            assert L.anni_f32_to_bf16(buf.ptr, stage.ptr, n) == 0
+        elif grad_type == 2:
+            sc = DeviceBuffer(len(tensors) * 4)
+            for i, (off, cnt) in enumerate(zip(opt.offsets, opt.sizes)):
+                assert L.anni_fp8_quantize(buf.ptr + off, sc.ptr + 4 * i, stage.ptr + 4 * off,
+                                           cnt) == 0
+        assert L.gpu_stream_sync() == 0
+        ring.append(buf)
+        scales.append(sc)
+    return ring, scales
+
+
+def cpu_baselines(size_name, norm_bpp, upd_bpp, budget_s):
+    """The step on the host cores of this box: (multithreaded port, single-thread reference)."""
+    from anni_amd import layout
+    from oracle import binding as ob
+    ob.lib()
+    threads = min(ob.lib().oracle_max_threads(), len(os.sched_getaffinity(0)))
+    n_full = layout.param_count(size_name)
+    bpp = norm_bpp + upd_bpp
+    rng = np.random.default_rng(0)
+
+    def sample(n):
+        p = (rng.standard_normal(n, dtype=np.float32) * np.float32(0.02))
+        g0 = (rng.standard_normal(n, dtype=np.float32) * np.float32(1e-3))
+        return p, g0
+
+    # multithreaded restatement, SoA, all cores; norm by ordered partials
+    n = min(n_full, 48 << 20)
+    p, g0 = sample(n)
+    m = np.zeros(n, np.float32)
+    v = np.zeros(n, np.float32)
+    O = ob.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, threads=threads,
+                  norm_threads=threads)
+    g = g0.copy()
+    O.step(p, g, m, v, 3e-6, 1.0 / (math.sqrt(n) * 1e-3) * 1.7)      # warm the pages
+    times = []
+    t_end = time.perf_counter() + budget_s * 0.5
+    k = 0
+    while k < 3 or (time.perf_counter() < t_end and k < 12):
+        g[:] = g0
+        gs = 1.0 / (math.sqrt(n) * 1e-3) * (1.7 if k % 2 else 0.6)
+        t0 = time.perf_counter()
+        O.step(p, g, m, v, 3e-6 * (k + 2), gs)
+        times.append(time.perf_counter() - t0)
+        k += 1
+    mt = float(np.median(times))
+    mt_out = {
+        "value": round(n * bpp / mt / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": "first %d of %d params of the workload, %d timed steps (median), fp32 state, "
+                  "clip 1.0 + decay 0.1, OpenMP over %d threads" % (n, n_full, len(times), threads),
+        "params_per_s": round(n / mt, 1), "ms_per_step_sample": round(mt * 1e3, 3),
+        "ms_per_step_extrapolated": round(mt * 1e3 * n_full / n, 1),
+    }
+    del p, g, g0, m, v
+
+    # the reference's own serial loop (compiled reference if it travelled, else the slot-layout port)
+    n = min(n_full, 12 << 20)
+    p, g0 = sample(n)
+    g = g0.copy()
+    if ob.ref_available():
+        R = ob.RefAdam(p, g, beta2=0.95, weight_decay=0.1, grad_clip=1.0)
+        kind = "reference"
+
+        def one(k):
+            R.step(3e-6 * (k + 1), 1.0 / (math.sqrt(n) * 1e-3) * (1.7 if k % 2 else 0.6))
+    else:
+        kind = "port"
+        slots = np.zeros(n, dtype=[("param", np.uint64), ("grad", np.uint64), ("m", np.float32),
+                                   ("v", np.float32)])
+        slots["param"] = p.ctypes.data + 4 * np.arange(n, dtype=np.uint64)
+        slots["grad"] = g.ctypes.data + 4 * np.arange(n, dtype=np.uint64)
+
+        def one(k):
+            ob.lib().oracle_adam_step_slots(
+                slots.ctypes.data, n, k + 1, 0.9, 0.95, 1e-8, 0.1, 1.0, 3e-6 * (k + 1),
+                1.0 / (math.sqrt(n) * 1e-3) * (1.7 if k % 2 else 0.6))
+    one(0)
+    times = []
+    for k in range(1, 4):
+        g[:] = g0
+        t0 = time.perf_counter()
+        one(k)
+        times.append(time.perf_counter() - t0)
+    st = float(np.median(times))
+    serial_out = {
+        "value": round(n * bpp / st / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": kind,
+        "sample": "first %d of %d params, 3 timed steps (median), the reference's serial "
+                  "24-byte-slot loop" % (n, n_full),
+        "params_per_s": round(n / st, 1), "ns_per_param": round(st / n * 1e9, 3),
+        "ms_per_step_extrapolated": round(st * 1e3 * n_full / n, 1),
+    }
+    return mt_out, serial_out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="555m", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
+    ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds for the CPU legs")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (the step has no multi-GPU path); "
+                 "use --gpus 1")
+    if a.steps < 1 or a.warmup < 0:
+        sys.exit("bench.py: --steps >= 1 and --warmup >= 0")
+
+    from anni_amd import layout, lib
+    from anni_amd.lm_adam import LmAdam
+    L = lib.require_gpu()
+
+    size, gt, mt, norm_bpp, upd_bpp = WORKLOADS[a.workload]
+    tensors = layout.tensors(size)
+    opt = LmAdam(tensors, grad_type=gt, moment_type=mt, twins=True, skip_nonfinite=True,
+                 own_grad=False, beta2=0.95, weight_decay=0.1, grad_clip=1.0)
+    n = opt.n
+    assert L.anni_fill_normal_f32(opt.o.d_param, n, 20260101, 1, 0.0, 0.02) == 0
+    opt.seed_twins()
+    total = a.steps + a.warmup
+    ring, scales = make_grad_ring(L, opt, tensors, total, gt, 20260101)
+
+    # per-step inputs: warmup(100)+cosine lr at schedule steps 0.., grad scale straddling the clip
+    from anni_amd import lm_adam
+    lrs = [lm_adam.step_lr(3e-4, s, 100, 1000, "cosine") for s in range(total)]
+    unit = 1.0 / (math.sqrt(n) * 1e-3)
+    gss = [unit * (1.7 if s % 2 else 0.6) for s in range(total)]
+
+    def run(first, count, per_kernel):
+        ptrs = (C.c_void_p * count)(*[ring[first + i].ptr for i in range(count)])
+        lr = (C.c_double * count)(*lrs[first:first + count])
+        gs = (C.c_double * count)(*gss[first:first + count])
+        ms, ms_a, ms_b = C.c_float(0), C.c_float(0), C.c_float(0)
+        if gt == 2:
+            # fp8: each flat carries its own per-tensor scales -> one call per step
+            tot = sa = sb = 0.0
+            for i in range(count):
+                opt.o.d_gscale = scales[first + i].ptr
+                one = (C.c_void_p * 1)(ptrs[i])
+                rc = L.anni_adam_time_steps(opt.h, 1, one, 1, C.byref(C.c_double(lr[i])),
+                                            C.byref(C.c_double(gs[i])), C.byref(ms),
+                                            C.byref(ms_a) if per_kernel else None,
+                                            C.byref(ms_b) if per_kernel else None)
+                assert rc == 0, L.gpu_debug_last_error()
+                tot, sa, sb = tot + ms.value, sa + ms_a.value, sb + ms_b.value
+            return tot, sa, sb
+        rc = L.anni_adam_time_steps(opt.h, count, ptrs, count, lr, gs, C.byref(ms),
+                                    C.byref(ms_a) if per_kernel else None,
+                                    C.byref(ms_b) if per_kernel else None)
+        assert rc == 0, L.gpu_debug_last_error()
+        return ms.value, ms_a.value, ms_b.value
+
+    if a.warmup:
+        run(0, a.warmup, False)
+    L.gpu_device_sync()
+    t0 = time.perf_counter()
+    ev_ms, ms_sumsq, ms_update = run(a.warmup, a.steps, True)
+    L.gpu_device_sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+
+    st = opt.sync_stats()
+    assert opt.t == total and math.isfinite(st.last_grad_norm)
+    bpp = norm_bpp + upd_bpp
+    ms_step = wall_ms / a.steps
+    step_gbps = n * bpp / (ms_step * 1e-3) / 1e9
+    upd_ms = ms_update / a.steps
+    sumsq_ms = ms_sumsq / a.steps
+    upd_gbps = n * upd_bpp / (upd_ms * 1e-3) / 1e9
+    out = {
+        "metric": "AdamW step HBM GB/s (algorithmic bytes / step time; AdamW + global-norm clip "
+                  "+ decay + bf16 twins), %s param set" % a.workload,
+        "value": round(step_gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f64",
+        "data": "synthetic",
+        "config": {"workload": a.workload, "storage": STORAGE[a.workload], "params": n, "tensors": len(tensors),
+                   "bytes_per_param": bpp, "clip": 1.0, "weight_decay": 0.1, "beta2": 0.95,
+                   "lr": "3e-4 warmup100+cosine", "twins": "bf16 RNE on matrices",
+                   "launches_per_step": 2},
+        "params_per_s": round(n / (ms_step * 1e-3), 1),
+        "pct_of_hbm_peak": round(100.0 * step_gbps / HBM_PEAK_GBPS, 2),
+        "event_ms_per_step": round(ev_ms / a.steps, 4),
+        "roofline": {"bound": "hbm", "kernel": "adam_update_kernel", "achieved": round(upd_gbps, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(upd_gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "bytes_per_launch": n * upd_bpp, "avg_ms": round(upd_ms, 4)},
+        "sumsq_kernel": {"avg_ms": round(sumsq_ms, 4), "bytes_per_launch": n * norm_bpp,
+                         "achieved": round(n * norm_bpp / (sumsq_ms * 1e-3) / 1e9, 1)
+                         if sumsq_ms > 0 else None, "unit": "GB/s"},
+        "last_grad_norm": st.last_grad_norm, "last_clipped": int(st.last_clipped),
+    }
+    if not a.no_cpu:
+        mt_out, serial_out = cpu_baselines(size, norm_bpp, upd_bpp, a.cpu_budget)
+        out["cpu_baseline"] = mt_out
+        out["cpu_reference_serial"] = serial_out
+        out["gpu_over_cpu"] = round(step_gbps / mt_out["value"], 1)
+    print(json.dumps(out))
+    opt.free()
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,153 @@
+/*
+** anni_adam.h -- device-resident AdamW optimizer over a multi-tensor flat, the
+** MI355X counterpart of the reference's lang/lm_adam.{h,c}.
+**
+** What the reference's flat ABI (num/gpu.h:121-132) cannot express is added
+** here: weight decay on selected tensors only, bf16-stored moments, bf16 or
+** fp8-E4M3 gradients with a per-tensor scale, the clip norm and the non-finite
+** skip decided on the device without a host round trip, and a launch table that
+** covers every tensor -- matrices, embeddings, biases, LayerNorm vectors -- in
+** one sum-of-squares launch and one update launch per step.
+**
+** The struct mirrors the public fields of the reference's lm_adam
+** (lang/lm_adam.h:30-54): callers set beta1/beta2/eps/weight_decay/grad_clip
+** directly and read t / last_grad_norm, as lang/lm_train.c:1336-1351 does.
+**
+** Arithmetic: the reference's host loop (lang/lm_adam.c:571-598) -- double
+** intermediates, float stores after m, v, the step and the decay -- so the FP32
+** state equals the CPU path bit for bit under the same effective gradient
+** scale; the twins are round-to-nearest-even bf16 of the final p
+** (num/gpu_cuda.cu:8578).
+**
+** Results: 0 = done, -1 = failed (bad argument, no device, launch error); no
+** CPU fallback exists in this library.
+*/
+#ifndef ANNI_ADAM_H__
+#define ANNI_ADAM_H__
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element storage types. */
+#define ANNI_F32	0
+#define ANNI_BF16	1	/* upper 16 bits of an IEEE float */
+#define ANNI_FP8_E4M3	2	/* OCP E4M3: bias 7, max 448, S.1111.111 = NaN, no infinities */
+
+/* Tensor flags. */
+#define ANNI_T_DECAY	1u	/* decoupled weight decay applies (BASELINE: matrices only) */
+#define ANNI_T_TWIN	2u	/* the bf16 twin of this tensor is written */
+
+/* One registered tensor; tensors are packed in registration order with no padding (lm_adam.c:25-57). */
+typedef struct anni_tensor {
+	int64_t		n;
+	uint32_t	flags;
+} anni_tensor;
+
+typedef struct anni_adam_config {
+	int	grad_type;	/* ANNI_F32 / ANNI_BF16 / ANNI_FP8_E4M3 */
+	int	moment_type;	/* ANNI_F32 / ANNI_BF16 (computed in double, rounded f32 then bf16 on store) */
+	int	twins;		/* 1: allocate the bf16 twin flat */
+	int	skip_nonfinite;	/* 1: a non-finite gradient norm skips the update (lm_adam.c:474-483) */
+	int	own_grad;	/* 1: the arena allocates the gradient flat; 0: bind one with anni_adam_bind_grad */
+} anni_adam_config;
+
+struct anni_adam_priv;
+
+typedef struct anni_adam {
+	int64_t	n;		/* elements in the flat */
+	int	n_tensors;
+	int	t;		/* steps taken (advanced by every step with lr > 0, lm_adam.c:531-533) */
+	double	beta1;		/* defaults 0.9, 0.999, 1e-8, 0, 0 (lm_adam.c:110-115) */
+	double	beta2;
+	double	eps;
+	double	weight_decay;
+	double	grad_clip;	/* global L2 clip; 0 = off */
+	double	last_sumsq;	/* valid after anni_adam_sync_stats */
+	double	last_grad_norm;
+	double	last_grad_scale;
+	int	last_skipped;
+	int	last_clipped;
+	anni_adam_config cfg;
+	/* the device arena: one allocation, each flat 2 MiB aligned */
+	float	*d_param;
+	void	*d_param_bf16;
+	void	*d_grad;
+	void	*d_m;
+	void	*d_v;
+	float	*d_gscale;	/* per-tensor fp8 dequant scale (n_tensors floats) */
+	struct anni_adam_priv *priv;
+} anni_adam;
+
+/*
+** Counterpart of lm_adam_create + gpu_buffers_init (lm_adam.c:79-139,217-311):
+** registers the tensors in order at packed offsets, allocates the arena (p, m,
+** v zeroed; gradients zeroed when own_grad), builds the launch table.
+** NULL on failure.
+*/
+anni_adam	*anni_adam_create(const anni_tensor *tensors, int n_tensors,
+			const anni_adam_config *cfg);
+/* lm_adam_free (lm_adam.c:185-194). */
+void	anni_adam_free(anni_adam **opt);
+/* Element offset of tensor i in every flat. */
+int64_t	anni_adam_tensor_offset(const anni_adam *opt, int i);
+/* Use an external gradient flat (n elements of grad_type, e.g. written by backward). */
+int	anni_adam_bind_grad(anni_adam *opt, void *d_grad);
+/* gpu_adam_seed_bf16_flat: twins = bf16(p) for the whole flat (after loading weights). */
+int	anni_adam_seed_twins(anni_adam *opt);
+/* lm_adam_zero_grad: clears the gradient flat on the stream. */
+int	anni_adam_zero_grad(anni_adam *opt);
+/*
+** lm_adam_step_scaled (lm_adam.c:522-607): lr <= 0 returns 1 without advancing t;
+** otherwise t++, [sum of squares when grad_clip > 0 or skip_nonfinite], update.
+** Asynchronous on the compute stream: nothing is read back.
+*/
+int	anni_adam_step_scaled(anni_adam *opt, double lr, double grad_scale);
+/* lm_adam_step. */
+int	anni_adam_step(anni_adam *opt, double lr);
+/* Waits for the stream and fills last_sumsq / last_grad_norm / last_grad_scale / last_skipped / last_clipped. */
+int	anni_adam_sync_stats(anni_adam *opt);
+
+/* lm_train_step_lr and its setters (lang/lm_train.c:98-124,398-411); kind "none" / "linear" / "cosine". */
+void	anni_lr_set_schedule(int warmup_steps, int decay_steps, const char *kind);
+void	anni_lr_set_sched_from(int from);
+double	anni_lr_step(double base_lr, int step);
+
+/* ---- stream plumbing ---------------------------------------------------- */
+
+/* The compute stream (a hipStream_t); anni_gpu_set_stream(NULL) restores the library's own. */
+void	*anni_gpu_stream(void);
+void	anni_gpu_set_stream(void *hip_stream);
+
+/*
+** Times `count` back-to-back steps with HIP events recorded on the compute
+** stream: per step, the gradient flat grads[i % n_grads] is bound (NULL array =
+** keep the bound one), lr[i] and grad_scale[i] are used.  ms_total receives the
+** elapsed time of the whole run, ms_sumsq / ms_update (may be NULL) the summed
+** durations of the two kernels.  Allocates nothing on the device.
+*/
+int	anni_adam_time_steps(anni_adam *opt, int count, void *const *grads, int n_grads,
+		const double *lr, const double *grad_scale, float *ms_total,
+		float *ms_sumsq, float *ms_update);
+
+/* ---- producers either side of the step (device utilities) ---------------- */
+
+/* x[i] = mean + std * N(0,1), counter-based (seed, stream, i): same values for any launch shape. */
+int	anni_fill_normal_f32(float *d_x, int64_t n, uint64_t seed, uint64_t stream,
+		float mean, float std);
+/* dst = bf16(src) round to nearest even (num/gpu_cuda.cu:1497-1513). */
+int	anni_f32_to_bf16(void *d_dst, const float *d_src, int64_t n);
+/*
+** Per-tensor FP8 quantisation by the reference's convention (num/gpu_cuda.cu:796-851,927-938):
+** scale = max(amax/448, 1e-12) (amax <= 0 or non-finite: 1e-8/448), q = satfinite_e4m3(x * (1/scale)).
+** d_scale[0] receives the scale; d_src is only read.
+*/
+int	anni_fp8_quantize(void *d_q, float *d_scale, const float *d_src, int64_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

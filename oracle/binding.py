@@ -1,0 +1,222 @@
+"""ctypes binding of the CPU oracle (liboracle.so) and, where it was built, of the
+reference's own compiled optimizer (oracle/_ref/libanni_ref.so).
+
+Test infrastructure only: imported by tests, by the smoke check and by the
+bench's cpu_baseline leg; never by the package that ships.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ORACLE_SO = os.path.join(HERE, "liboracle.so")
+REF_SO = os.path.join(HERE, "_ref", "libanni_ref.so")
+
+F32, BF16, FP8 = 0, 1, 2
+KIND = {"none": 0, "linear": 1, "cosine": 2}
+
+
+class Seg(C.Structure):
+    _fields_ = [("off", C.c_int64), ("n", C.c_int64), ("wd_on", C.c_int),
+                ("gscale", C.c_float)]
+
+
+class OracleAdam(C.Structure):
+    _fields_ = [("n", C.c_int64), ("t", C.c_int), ("beta1", C.c_double),
+                ("beta2", C.c_double), ("eps", C.c_double),
+                ("weight_decay", C.c_double), ("grad_clip", C.c_double),
+                ("skip_nonfinite", C.c_int), ("grad_type", C.c_int),
+                ("moment_type", C.c_int), ("norm_threads", C.c_int),
+                ("last_sumsq", C.c_double), ("last_grad_norm", C.c_double),
+                ("last_grad_scale", C.c_double), ("last_clipped", C.c_int),
+                ("last_skipped", C.c_int)]
+
+
+def build(force=False):
+    """Compile liboracle.so (and _ref when the reference tree is present)."""
+    if force or not os.path.exists(ORACLE_SO):
+        subprocess.check_call(["make", "-C", HERE, "-s"] + (["-B"] if force else []))
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(ORACLE_SO):
+            build()
+        L = C.CDLL(ORACLE_SO)
+        L.oracle_adam_defaults.argtypes = [C.POINTER(OracleAdam), C.c_int64]
+        L.oracle_adam_step_scaled.argtypes = [
+            C.POINTER(OracleAdam), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+            C.c_void_p, C.POINTER(Seg), C.c_int, C.c_double, C.c_double,
+            C.POINTER(C.c_double), C.c_int]
+        L.oracle_adam_step_scaled.restype = C.c_int
+        L.oracle_sumsq.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.POINTER(Seg),
+                                   C.c_int, C.c_double, C.c_int]
+        L.oracle_sumsq.restype = C.c_double
+        L.oracle_lr.argtypes = [C.c_double, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+        L.oracle_lr.restype = C.c_double
+        L.oracle_bf16_rne.argtypes = [C.c_float]
+        L.oracle_bf16_rne.restype = C.c_uint16
+        L.oracle_fp8_decode.argtypes = [C.c_uint8]
+        L.oracle_fp8_decode.restype = C.c_float
+        L.oracle_fp8_encode.argtypes = [C.c_float]
+        L.oracle_fp8_encode.restype = C.c_uint8
+        L.oracle_fp8_scale_from_amax.argtypes = [C.c_float]
+        L.oracle_fp8_scale_from_amax.restype = C.c_float
+        L.oracle_fp8_quantize.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+        L.oracle_fp8_quantize.restype = C.c_float
+        L.oracle_f32_to_bf16.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+        L.oracle_adam_step_slots.argtypes = [
+            C.c_void_p, C.c_int64, C.c_int, C.c_double, C.c_double, C.c_double,
+            C.c_double, C.c_double, C.c_double, C.c_double]
+        L.oracle_max_threads.restype = C.c_int
+        _lib = L
+    return _lib
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def make_segs(tensors):
+    """tensors: iterable of (off, n, wd_on, gscale) -> ctypes array."""
+    arr = (Seg * len(tensors))()
+    for i, (off, n, wd_on, gscale) in enumerate(tensors):
+        arr[i] = Seg(off, n, int(wd_on), float(gscale))
+    return arr
+
+
+class Oracle:
+    """Host optimizer state over flat numpy arrays, stepped by the C oracle."""
+
+    def __init__(self, n, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0,
+                 grad_clip=0.0, skip_nonfinite=False, grad_type=F32, moment_type=F32,
+                 tensors=None, threads=1, norm_threads=1):
+        self.o = OracleAdam()
+        lib().oracle_adam_defaults(C.byref(self.o), n)
+        self.o.beta1, self.o.beta2, self.o.eps = beta1, beta2, eps
+        self.o.weight_decay, self.o.grad_clip = weight_decay, grad_clip
+        self.o.skip_nonfinite = int(skip_nonfinite)
+        self.o.grad_type, self.o.moment_type = grad_type, moment_type
+        self.o.norm_threads = norm_threads
+        self.threads = threads
+        self.segs = make_segs(tensors) if tensors is not None else None
+        self.nsegs = len(tensors) if tensors is not None else 0
+
+    def set_gscales(self, scales):
+        for i, s in enumerate(scales):
+            self.segs[i].gscale = float(s)
+
+    def step(self, p, g, m, v, lr, grad_scale=1.0, twin=None, sumsq_override=None):
+        ov = None
+        if sumsq_override is not None:
+            ov = C.byref(C.c_double(float(sumsq_override)))
+        return lib().oracle_adam_step_scaled(
+            C.byref(self.o), _ptr(p), _ptr(g), _ptr(m), _ptr(v), _ptr(twin),
+            self.segs, self.nsegs, lr, grad_scale, ov, self.threads)
+
+    @property
+    def t(self):
+        return self.o.t
+
+
+def sumsq(g, grad_type=F32, tensors=None, grad_scale=1.0, threads=1):
+    segs = make_segs(tensors) if tensors is not None else None
+    return lib().oracle_sumsq(_ptr(g), grad_type, g.size, segs,
+                              len(tensors) if tensors is not None else 0, grad_scale,
+                              threads)
+
+
+def lr(base_lr, step, warmup=0, decay_steps=0, kind="none", sched_from=0):
+    return lib().oracle_lr(base_lr, step, warmup, decay_steps, KIND[kind], sched_from)
+
+
+def bf16_rne(x):
+    """float32 array -> uint16 array (round to nearest even)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint16)
+    lib().oracle_f32_to_bf16(_ptr(out), _ptr(x), x.size)
+    return out
+
+
+def bf16_widen(h):
+    return (h.astype(np.uint32) << 16).view(np.float32)
+
+
+def fp8_decode_table():
+    return np.array([lib().oracle_fp8_decode(q) for q in range(256)], dtype=np.float32)
+
+
+def fp8_quantize(x):
+    """float32 tensor -> (uint8 codes, float scale) by the per-tensor amax convention."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    q = np.empty(x.shape, dtype=np.uint8)
+    scale = lib().oracle_fp8_quantize(_ptr(q), _ptr(x), x.size)
+    return q, np.float32(scale)
+
+
+# ---- the reference's own compiled optimizer (present only where it was built) ----
+
+_ref = None
+
+
+def ref_available():
+    return os.path.exists(REF_SO)
+
+
+def ref():
+    global _ref
+    if _ref is None:
+        R = C.CDLL(REF_SO)
+        R.ref_adam_create.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                      C.c_long, C.c_int, C.c_double, C.c_double,
+                                      C.c_double, C.c_double, C.c_double]
+        R.ref_adam_create.restype = C.c_void_p
+        R.ref_adam_step.argtypes = [C.c_void_p, C.c_double, C.c_double]
+        R.ref_adam_step.restype = C.c_int
+        R.ref_adam_set.argtypes = [C.c_void_p, C.c_double, C.c_double]
+        R.ref_adam_export.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        R.ref_adam_free.argtypes = [C.c_void_p]
+        R.ref_step_lr.argtypes = [C.c_double, C.c_int, C.c_int, C.c_int, C.c_char_p,
+                                  C.c_int]
+        R.ref_step_lr.restype = C.c_double
+        _ref = R
+    return _ref
+
+
+class RefAdam:
+    """The reference's lm_adam_step_scaled (host path) over flat numpy arrays."""
+
+    def __init__(self, p, g, m=None, v=None, t=0, beta1=0.9, beta2=0.999, eps=1e-8,
+                 weight_decay=0.0, grad_clip=0.0):
+        self.p, self.g = p, g
+        self.h = ref().ref_adam_create(_ptr(p), _ptr(g), _ptr(m), _ptr(v), p.size, t,
+                                       beta1, beta2, eps, weight_decay, grad_clip)
+        if not self.h:
+            raise MemoryError("ref_adam_create")
+
+    def step(self, lr, grad_scale=1.0):
+        return ref().ref_adam_step(self.h, lr, grad_scale)
+
+    def moments(self):
+        m = np.empty(self.p.size, dtype=np.float32)
+        v = np.empty(self.p.size, dtype=np.float32)
+        ref().ref_adam_export(self.h, _ptr(m), _ptr(v))
+        return m, v
+
+    def close(self):
+        if self.h:
+            ref().ref_adam_free(self.h)
+            self.h = None
+
+    def __del__(self):
+        self.close()
+
+
+def ref_lr(base_lr, step, warmup=0, decay_steps=0, kind="none", sched_from=0):
+    return ref().ref_step_lr(base_lr, step, warmup, decay_steps, kind.encode(), sched_from)

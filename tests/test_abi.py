@@ -1,0 +1,136 @@
+"""The C-ABI library loads, exports every declared symbol, and answers as the headers say when
+there is no device.  Host-only logic (the learning-rate schedule, the tensor layout) is checked
+here too.  No compute calls: runs without a GPU."""
+import ctypes as C
+import glob
+import os
+import re
+
+import numpy as np
+import pytest
+
+from helpers import GOLDEN
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    names = set()
+    for h in glob.glob(os.path.join(ROOT, "include", "*.h")):
+        text = open(h).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b((?:gpu|anni)_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
+
+
+def test_every_declared_symbol_is_exported():
+    from anni_amd import lib
+    L = C.CDLL(lib.SO_PATH)
+    syms = declared_symbols()
+    gpu = [s for s in syms if s.startswith("gpu_")]
+    assert len(gpu) == 99, len(gpu)          # the whole of num/gpu.h
+    for s in syms:
+        assert getattr(L, s) is not None, s
+    for s in lib._PROTOS:
+        assert s in syms, s
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from anni_amd import lib
+    monkeypatch.setattr(lib, "_lib", None)
+    monkeypatch.setattr(lib, "SO_PATH", "/nonexistent/libanni_gpu_hip.so")
+    with pytest.raises(lib.LibraryMissing):
+        lib.load()
+
+
+def _no_device(L):
+    return L.gpu_available() == 0
+
+
+def test_without_a_device_every_entry_declines():
+    from anni_amd import lib
+    L = lib.load()
+    if not _no_device(L):
+        pytest.skip("a device is present")
+    assert L.gpu_backend_name() == b"hip-gfx950"
+    assert L.gpu_malloc(1024) is None
+    assert L.gpu_host_alloc(1024) is None
+    buf = np.zeros(16, np.float32)
+    out = C.c_double(0)
+    assert L.gpu_grad_sumsq(buf.ctypes.data, 16, C.byref(out)) == -1
+    assert L.gpu_adam_step_dev_bf16(buf.ctypes.data, None, buf.ctypes.data, buf.ctypes.data,
+                                    buf.ctypes.data, 16, 1e-3, 0.9, 0.95, 1e-8, 1, 1.0) == -1
+    assert L.gpu_memcpy_h2d(buf.ctypes.data, buf.ctypes.data, 64) == -1
+    assert L.gpu_memset(buf.ctypes.data, 0, 64) == -1
+    assert L.gpu_stream_sync() == -1
+    assert L.gpu_adam_seed_bf16_flat(buf.ctypes.data, buf.ctypes.data, 16) == -1
+    L.gpu_device_sync()
+    L.gpu_free(None)
+    t = (lib.Tensor * 1)(lib.Tensor(16, 3))
+    cfg = lib.Config(0, 0, 1, 0, 1)
+    assert not L.anni_adam_create(t, 1, C.byref(cfg))
+    assert L.anni_adam_step_scaled(None, 1e-3, 1.0) == -1
+
+
+def test_unserved_symbols_answer_like_the_cpu_stub():
+    from anni_amd import lib
+    L = C.CDLL(lib.SO_PATH)
+    for name in ("gpu_mat_mul", "gpu_mat_mul_bt", "gpu_graph_begin", "gpu_graph_replay"):
+        fn = getattr(L, name)
+        fn.restype = C.c_int
+        assert fn(None, None, None) == -1
+    for name, want in (("gpu_fp8", 0), ("gpu_graph_supported", 0), ("gpu_graph_replayable", 0),
+                       ("gpu_ce_bias_fused", 0)):
+        fn = getattr(L, name)
+        fn.restype = C.c_int
+        assert fn() == want
+    L.gpu_attn_qkv_bwd.restype = C.c_int
+    assert L.gpu_attn_qkv_bwd(None, None, None, None, None, None, None, None, None) == 1
+    L.gpu_set_sync_mode(1)
+    assert L.gpu_sync_mode() == 1
+    L.gpu_set_sync_mode(0)
+    L.gpu_copy_stream.restype = C.c_void_p
+    assert L.gpu_copy_stream() is None
+
+
+def test_weight_epoch_moves_on_invalidate():
+    from anni_amd import lib
+    L = lib.load()
+    e0 = L.gpu_param_epoch()
+    L.gpu_half_wt_invalidate(None)
+    assert L.gpu_param_epoch() == e0 + 1
+
+
+def test_lr_schedule_host_logic(oracle):
+    from anni_amd import lm_adam
+    # the reference's own known answers (tests/test_ann.c:866-879)
+    f = lm_adam.step_lr
+    assert abs(f(1.0, 29000, 100, 1000, "cosine", 0) - 0.0) < 1e-12
+    assert abs(f(1.0, 29000, 100, 1000, "cosine", 29000) - 0.01) < 1e-12
+    assert abs(f(1.0, 29099, 100, 1000, "cosine", 29000) - 1.0) < 1e-12
+    assert abs(f(1.0, 29600, 100, 1000, "cosine", 29000) - 0.5) < 1e-12
+    assert abs(f(1.0, 31000, 100, 1000, "cosine", 29000) - 0.0) < 1e-12
+    assert abs(f(1.0, 10, 100, 1000, "cosine", 29000) - 0.01) < 1e-12
+    # the table the compiled reference wrote, and the oracle, bit for bit
+    T = np.load(os.path.join(GOLDEN, "lr_table.npz"))
+    for row, case in zip(T["lr"], T["cases"]):
+        w, d, k, frm = str(case).split(",")
+        for s, want in zip(T["steps"], row):
+            got = f(3e-4, int(s), int(w), int(d), k, int(frm))
+            assert got == want == oracle.lr(3e-4, int(s), int(w), int(d), k, int(frm))
+    # setters clamp negatives (lm_train.c:398-411)
+    assert f(1.0, 5, -3, -7, "cosine", -2) == 1.0
+
+
+def test_layout_parameter_counts():
+    from anni_amd import layout
+    assert layout.param_count("185m") == 167948288
+    assert layout.param_count("555m") == 555848096
+    assert layout.param_count("1p4b") == 1413498528
+    assert layout.param_count("185m", "reference") == 167899136
+    assert layout.param_count("555m", "reference") == 555762080
+    assert layout.param_count("1p4b", "reference") == 1413301920
+    assert len(layout.tensors("185m")) == 2 + 12 * 12
+    assert len(layout.tensors("555m", "reference")) == 2 + 12 * 14
+    mats = [t for t in layout.tensors("555m") if t[2]]
+    assert all(n >= 1536 * 1536 for _nm, n, _f in mats)

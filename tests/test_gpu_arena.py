@@ -1,0 +1,319 @@
+"""Parity of the multi-tensor arena step (include/anni_adam.h) against the CPU oracle, through the
+C ABI: BASELINE configurations at reduced size, ragged tensor lists, every storage mode, the
+non-finite skip, and the golden vectors of the reference."""
+import numpy as np
+import pytest
+
+from helpers import GOLDEN_CASES, load_golden, same_bits, rel_err, bf16_ulp_diff
+
+pytestmark = pytest.mark.gpu
+
+TOL_STATE = 1e-6     # BASELINE: FP32 master/m/v within 1e-6 relative per step
+TOL_NORM = 1e-5      # BASELINE: clip norm within 1e-5 relative
+
+F32, BF16, FP8 = 0, 1, 2
+DECAY, TWIN = 1, 2
+
+RAGGED = [(5000, 3), (3, 0), (4096, 3), (1, 2), (0, 3), (8191, 1), (12288, 3), (7, 0), (4097, 3),
+          (2, 1), (40000, 3), (1023, 0)]
+
+
+def oracle_tensors(opt, gscales=None):
+    return [(opt.offsets[i], opt.sizes[i], 1 if (f & DECAY) else 0,
+             1.0 if gscales is None else float(gscales[i]))
+            for i, f in enumerate(opt._flags)]
+
+
+def make(gpu, tensors, **kw):
+    from anni_amd.lm_adam import LmAdam
+    opt = LmAdam(tensors, **kw)
+    opt._flags = [t[-1] for t in tensors]
+    return opt
+
+
+def twin_mask(opt):
+    mask = np.zeros(opt.n, bool)
+    for off, n, f in zip(opt.offsets, opt.sizes, opt._flags):
+        if f & TWIN:
+            mask[off:off + n] = True
+    return mask
+
+
+def run_fp32_case(gpu, oracle, tensors, steps, clip, wd, gmul, grad_scale=1.0, seed=0,
+                  sched=(100, 1000, "cosine")):
+    """Ten steps on the arena vs the oracle twice: against the oracle's own (serial) norm with the
+    BASELINE tolerances, and bit for bit when the oracle is handed the device's sum of squares."""
+    from anni_amd import lm_adam
+    rng = np.random.default_rng(seed)
+    opt = make(gpu, tensors, beta2=0.95, weight_decay=wd, grad_clip=clip)
+    n = opt.n
+    p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    opt.upload("param", p0)
+    opt.seed_twins()
+    A = dict(p=p0.copy(), m=np.zeros(n, np.float32), v=np.zeros(n, np.float32))   # own norm
+    B = dict(p=p0.copy(), m=np.zeros(n, np.float32), v=np.zeros(n, np.float32))   # device norm
+    twinB = oracle.bf16_rne(p0)
+    segs = oracle_tensors(opt)
+    OA = oracle.Oracle(n, beta2=0.95, weight_decay=wd, grad_clip=clip, tensors=segs, threads=4)
+    OB = oracle.Oracle(n, beta2=0.95, weight_decay=wd, grad_clip=clip, tensors=segs, threads=4)
+    mask = twin_mask(opt)
+    n_clipped = 0
+    for s in range(steps):
+        g = (rng.standard_normal(n) * 1e-3 * gmul[s % len(gmul)]).astype(np.float32)
+        opt.upload("grad", g)
+        lr = lm_adam.step_lr(3e-4, opt.t, *sched)
+        assert lr == oracle.lr(3e-4, s, *sched)
+        assert opt.step_scaled(lr, grad_scale) == 0
+        st = opt.sync_stats()
+        assert opt.t == s + 1
+        gA, gB = g.copy(), g.copy()
+        OA.step(A["p"], gA, A["m"], A["v"], lr, grad_scale)
+        p, m, v = opt.download("param"), opt.download("m"), opt.download("v")
+        tw, gd = opt.download("twin"), opt.download("grad")
+        if clip > 0:
+            assert abs(st.last_grad_norm - OA.o.last_grad_norm) <= TOL_NORM * OA.o.last_grad_norm
+            assert st.last_clipped == OA.o.last_clipped and st.last_skipped == 0
+            n_clipped += st.last_clipped
+        assert rel_err(p, A["p"]) <= TOL_STATE, s
+        assert rel_err(m, A["m"]) <= TOL_STATE and rel_err(v, A["v"]) <= TOL_STATE, s
+        assert bf16_ulp_diff(tw[mask], oracle.bf16_rne(A["p"])[mask]) <= 1
+        assert not gd.any()
+        OB.step(B["p"], gB, B["m"], B["v"], lr, grad_scale, twin=twinB,
+                sumsq_override=st.last_sumsq if clip > 0 else None)
+        assert same_bits(p, B["p"]) and same_bits(m, B["m"]) and same_bits(v, B["v"]), s
+        assert (tw[mask] == twinB[mask]).all()
+        assert (tw[~mask] == oracle.bf16_rne(p0)[~mask]).all()       # unflagged tensors keep the seed
+        if clip > 0:
+            assert st.last_grad_scale == OB.o.last_grad_scale
+    opt.free()
+    return n_clipped
+
+
+def test_config1_no_clip_ragged(gpu, oracle):
+    """BASELINE config 1 hyper-parameters (constant lr, no clip, decay on flagged tensors)."""
+    run_fp32_case(gpu, oracle, RAGGED, 10, clip=0.0, wd=0.1, gmul=[1.0], sched=(0, 0, "none"))
+
+
+def test_config2_clip_half_the_steps_ragged(gpu, oracle):
+    """BASELINE config 2: clip 1.0 with about half the steps clipping, warmup 100 + cosine."""
+    n = sum(t[0] for t in RAGGED)
+    base = 1.0 / (np.sqrt(n) * 1e-3)                       # gmul = base -> norm ~ 1
+    k = run_fp32_case(gpu, oracle, RAGGED, 10, clip=1.0, wd=0.1,
+                      gmul=[0.5 * base, 2.0 * base, 0.7 * base, 1.5 * base])
+    assert k == 5
+
+
+def test_tiny_model_layout_with_grad_scale(gpu, oracle):
+    """The reference's 64-wide test model and rig constants (tests/test_gpu.c:30-34,67-84)."""
+    from anni_amd import layout
+    t = layout.tensors("tiny", "reference")
+    k = run_fp32_case(gpu, oracle, t, 4, clip=1.0, wd=0.1, gmul=[300.0, 90000.0],
+                      grad_scale=1.0 / (4 * 63), sched=(0, 0, "none"), seed=1234)
+    assert k == 2
+
+
+def test_single_tensor_and_unit_sizes(gpu, oracle):
+    for tensors in ([(1, 3)], [(4095, 3)], [(4096, 3)], [(4097, 1)], [(1, 0)] * 9, [(0, 3), (5, 3), (0, 0)]):
+        run_fp32_case(gpu, oracle, tensors, 3, clip=1.0, wd=0.1, gmul=[1e3, 1.0], seed=len(tensors))
+
+
+def test_golden_vectors_through_arena(gpu, oracle):
+    """The reference's own outputs vs the fused device step (CPU-form clip, device norm)."""
+    from anni_amd.lm_adam import LmAdam
+    for name in GOLDEN_CASES:
+        G = load_golden(name)
+        n = G["p0"].size
+        opt = LmAdam([(n, 3)], beta1=float(G["beta1"]), beta2=float(G["beta2"]),
+                     eps=float(G["eps"]), weight_decay=float(G["wd"]), grad_clip=float(G["clip"]))
+        opt.upload("param", G["p0"])
+        exact = 0
+        for s in range(G["grads"].shape[0]):
+            opt.upload("grad", G["grads"][s])
+            assert opt.step_scaled(float(G["lr"][s]), float(G["grad_scale"])) == 0
+            p, m, v = opt.download("param"), opt.download("m"), opt.download("v")
+            assert rel_err(p, G["p"][s]) <= TOL_STATE and rel_err(m, G["m"][s]) <= TOL_STATE
+            assert rel_err(v, G["v"][s]) <= TOL_STATE
+            exact += same_bits(p, G["p"][s]) and same_bits(m, G["m"][s]) and same_bits(v, G["v"][s])
+            assert not opt.download("grad").any()
+        if float(G["clip"]) == 0.0:
+            assert exact == G["grads"].shape[0]              # no norm involved: bit for bit
+        opt.free()
+
+
+def test_lr_nonpositive_is_a_noop(gpu):
+    opt = make(gpu, [(100, 3)])
+    opt.upload("grad", np.ones(100, np.float32))
+    assert opt.step_scaled(0.0) == 1 and opt.t == 0          # lm_adam.c:531-532
+    assert opt.step_scaled(-1.0) == 1 and opt.t == 0
+    assert opt.download("grad").all() and not opt.download("param").any()
+    opt.free()
+
+
+@pytest.mark.parametrize("bad,where", [(np.nan, 0), (np.inf, 5000 + 3 + 17), (-np.inf, -1)])
+def test_nonfinite_skip_leaves_state_bit_identical(gpu, oracle, bad, where):
+    rng = np.random.default_rng(31)
+    opt = make(gpu, RAGGED, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True)
+    n = opt.n
+    p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    opt.upload("param", p0)
+    opt.seed_twins()
+    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True,
+                      tensors=oracle_tensors(opt), threads=4)
+    P, M, V = p0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    for s in range(4):
+        g = (rng.standard_normal(n) * 3e-3).astype(np.float32)
+        if s == 2:
+            g[where] = bad
+        before = [opt.download(k) for k in ("param", "m", "v", "twin")]
+        opt.upload("grad", g)
+        assert opt.step_scaled(1e-3) == 0
+        st = opt.sync_stats()
+        gg = g.copy()
+        O.step(P, gg, M, V, 1e-3, sumsq_override=st.last_sumsq if s != 2 else None)
+        assert st.last_skipped == O.o.last_skipped == (1 if s == 2 else 0)     # decision matches exactly
+        assert opt.t == O.t == s + 1                                            # t advances on a skip
+        after = [opt.download(k) for k in ("param", "m", "v", "twin")]
+        if s == 2:
+            for a, b in zip(before, after):
+                assert same_bits(a, b) if a.dtype == np.float32 else (a == b).all()
+        assert same_bits(after[0], P) and same_bits(after[1], M) and same_bits(after[2], V)
+        assert not opt.download("grad").any()
+    opt.free()
+
+
+def test_without_skip_flag_nonfinite_poisons_like_the_cpu_path(gpu, oracle):
+    """The reference's host loop has no skip: a NaN gradient reaches the state (lm_adam.c:571-598)."""
+    opt = make(gpu, [(4096, 3)], grad_clip=1.0)
+    g = np.full(4096, 1e-3, np.float32)
+    g[5] = np.nan
+    opt.upload("grad", g)
+    opt.step_scaled(1e-3)
+    st = opt.sync_stats()
+    assert st.last_skipped == 0 and np.isnan(st.last_grad_norm)
+    assert np.isnan(opt.download("param")[5])
+    opt.free()
+
+
+def test_bf16_moments_and_grads(gpu, oracle):
+    """BASELINE config 4 at reduced size, long tail included (parity unpinned by the reference:
+    the oracle defines the rounding points)."""
+    rng = np.random.default_rng(44)
+    opt = make(gpu, RAGGED, grad_type=BF16, moment_type=BF16, beta2=0.95, weight_decay=0.1,
+               grad_clip=1.0)
+    n = opt.n
+    p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    opt.upload("param", p0)
+    P = p0.copy()
+    M = np.zeros(n, np.uint16)
+    V = np.zeros(n, np.uint16)
+    twin = oracle.bf16_rne(p0)
+    opt.seed_twins()
+    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, grad_type=oracle.BF16,
+                      moment_type=oracle.BF16, tensors=oracle_tensors(opt), threads=4)
+    mask = twin_mask(opt)
+    base = 1.0 / (np.sqrt(n) * 1e-3)
+    for s in range(10):
+        g = oracle.bf16_rne((rng.standard_normal(n) * 1e-3 * base * (0.6 if s % 2 else 1.7))
+                            .astype(np.float32))
+        opt.upload("grad", g)
+        lr = oracle.lr(3e-4, s, 100, 1000, "cosine")
+        opt.step_scaled(lr)
+        st = opt.sync_stats()
+        own = oracle.sumsq(g, oracle.BF16)
+        assert abs(st.last_sumsq - own) <= 1e-12 * own
+        gg = g.copy()
+        O.step(P, gg, M, V, lr, twin=twin, sumsq_override=st.last_sumsq)
+        assert st.last_clipped == O.o.last_clipped == (0 if s % 2 else 1)
+        assert same_bits(opt.download("param"), P)
+        assert (opt.download("m") == M).all() and (opt.download("v") == V).all()
+        assert (opt.download("twin")[mask] == twin[mask]).all()
+        assert not opt.download("grad").any()
+    opt.free()
+
+
+def test_fp8_gradients_with_per_tensor_scale_and_skip(gpu, oracle):
+    """BASELINE config 5 at reduced size: device quantisation, in-kernel unscale, NaN skip."""
+    rng = np.random.default_rng(55)
+    tensors = [(6000, 3), (64, 0), (4096, 3), (8192 + 3, 3), (1, 0), (20000, 3)]
+    opt = make(gpu, tensors, grad_type=FP8, beta2=0.95, weight_decay=0.1, grad_clip=1.0,
+               skip_nonfinite=True)
+    n = opt.n
+    p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    opt.upload("param", p0)
+    opt.seed_twins()
+    P, M, V = p0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    twin = oracle.bf16_rne(p0)
+    mask = twin_mask(opt)
+    from anni_amd.lm_adam import DeviceBuffer
+    stage = DeviceBuffer(n * 4)
+    base = 1.0 / (np.sqrt(n) * 1e-3)
+    for s in range(6):
+        g32 = (rng.standard_normal(n) * 1e-3 * base * (0.5 if s % 2 else 2.0)).astype(np.float32)
+        for i, (off, cnt) in enumerate(zip(opt.offsets, opt.sizes)):
+            g32[off:off + cnt] *= 1.0 + i                   # different amax per tensor
+        if s == 3:
+            g32[opt.offsets[3] + 11] = np.nan               # one tensor carries a NaN
+        stage.upload(g32)
+        q_want = np.empty(n, np.uint8)
+        scales = np.empty(len(tensors), np.float32)
+        for i, (off, cnt) in enumerate(zip(opt.offsets, opt.sizes)):
+            assert gpu.anni_fp8_quantize(opt.o.d_grad + off, opt.o.d_gscale + 4 * i,
+                                         stage.ptr + 4 * off, cnt) == 0
+            q_want[off:off + cnt], scales[i] = oracle.fp8_quantize(g32[off:off + cnt])
+        assert gpu.gpu_stream_sync() == 0
+        q = opt.download("grad")
+        assert (q == q_want).all()                          # device quantiser == oracle quantiser
+        assert same_bits(opt.download("gscale"), scales)
+        O = None
+        lr = oracle.lr(3e-4, s, 100, 1000, "cosine")
+        opt.step_scaled(lr)
+        st = opt.sync_stats()
+        if O is None:
+            O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True,
+                              grad_type=oracle.FP8, tensors=oracle_tensors(opt, scales), threads=4)
+            O.o.t = s
+        qq = q.copy()
+        O.step(P, qq, M, V, lr, twin=twin, sumsq_override=None if s == 3 else st.last_sumsq)
+        assert st.last_skipped == O.o.last_skipped == (1 if s == 3 else 0)
+        if s != 3:
+            own = oracle.sumsq(q, oracle.FP8, oracle_tensors(opt, scales))
+            assert abs(st.last_sumsq - own) <= 1e-12 * own
+            assert st.last_clipped == O.o.last_clipped == (0 if s % 2 else 1)
+        assert same_bits(opt.download("param"), P) and same_bits(opt.download("m"), M)
+        assert same_bits(opt.download("v"), V)
+        assert (opt.download("twin")[mask] == twin[mask]).all()
+        assert not opt.download("grad").any()
+        assert opt.t == s + 1
+    opt.free()
+
+
+def test_fp8_decode_all_codes_on_device(gpu, oracle):
+    """Every E4M3 byte through the kernel's decoder: with m = v = 0 and t = 1, m = (1-b1) * g."""
+    opt = make(gpu, [(256, 0)], grad_type=FP8, beta1=0.5, beta2=0.5)
+    q = np.arange(256, dtype=np.uint8)
+    opt.upload("grad", q)
+    opt.upload("gscale", np.array([0.25], np.float32))
+    opt.step_scaled(1e-3)
+    m = opt.download("m")
+    want = (oracle.fp8_decode_table() * np.float32(0.25)).astype(np.float64) * 0.5
+    nan = np.isnan(want)
+    assert (np.isnan(m) == nan).all() and nan.sum() == 2
+    assert same_bits(m[~nan], want[~nan].astype(np.float32))
+    opt.free()
+
+
+def test_device_normal_generator_and_bf16_convert(gpu, oracle):
+    from anni_amd.lm_adam import DeviceBuffer
+    n = 1 << 20
+    a = DeviceBuffer(n * 4)
+    b = DeviceBuffer(n * 4)
+    assert gpu.anni_fill_normal_f32(a.ptr, n, 7, 3, 0.0, 1e-3) == 0
+    assert gpu.anni_fill_normal_f32(b.ptr, n, 7, 3, 0.0, 1e-3) == 0
+    x, y = a.download(np.float32, n), b.download(np.float32, n)
+    assert same_bits(x, y) and np.isfinite(x).all()
+    assert abs(x.mean()) < 5e-6 and abs(x.std() - 1e-3) < 1e-5
+    assert gpu.anni_fill_normal_f32(b.ptr, n, 7, 4, 0.0, 1e-3) == 0
+    assert not same_bits(x, b.download(np.float32, n))
+    h = DeviceBuffer(n * 2)
+    assert gpu.anni_f32_to_bf16(h.ptr, a.ptr, n) == 0
+    assert (h.download(np.uint16, n) == oracle.bf16_rne(x)).all()

@@ -1,0 +1,311 @@
+"""Parity of the flat drop-in ABI (the num/gpu.h entry points lang/lm_adam.c calls) against the
+CPU oracle, through the C ABI.  Bit-exact where the arithmetic is identical by construction;
+BASELINE tolerances (1e-6 relative on p/m/v, 1 bf16 ulp on twins, 1e-5 on the norm) where the
+summation order of the norm differs."""
+import ctypes as C
+import math
+
+import numpy as np
+import pytest
+
+from helpers import GOLDEN_CASES, load_golden, same_bits, rel_err, bf16_ulp_diff
+
+pytestmark = pytest.mark.gpu
+
+TOL_STATE = 1e-6     # BASELINE: FP32 master/m/v within 1e-6 relative per step
+TOL_NORM = 1e-5      # BASELINE: clip norm within 1e-5 relative
+
+
+def dev(gpu, arr):
+    from anni_amd.lm_adam import DeviceBuffer
+    arr = np.ascontiguousarray(arr)
+    b = DeviceBuffer(max(arr.nbytes, 16))
+    if arr.nbytes:
+        b.upload(arr)
+    return b
+
+
+def test_device_is_gfx950_backend(gpu):
+    assert gpu.gpu_available() == 1
+    assert gpu.gpu_backend_name() == b"hip-gfx950"
+    f, t = C.c_size_t(0), C.c_size_t(0)
+    assert gpu.gpu_mem_info(C.byref(f), C.byref(t)) == 0 and 0 < f.value <= t.value
+    assert gpu.gpu_debug_last_error() == b""
+
+
+def test_memory_primitives(gpu):
+    from anni_amd.lm_adam import DeviceBuffer
+    rng = np.random.default_rng(1)
+    x = rng.integers(0, 255, 100003, dtype=np.uint8)
+    a = dev(gpu, x)
+    b = DeviceBuffer(x.nbytes)
+    assert gpu.gpu_memcpy_d2d(b.ptr, a.ptr, x.nbytes) == 0
+    assert (b.download(np.uint8, x.size) == x).all()
+    # byte fill on awkward offsets / lengths, neighbours untouched
+    for off, ln, val in ((0, 100003, 0), (1, 17, 0xab), (3, 4099, 0x5c), (15, 1, 1), (16, 64, 0xff),
+                         (7, 99990, 0x11)):
+        assert gpu.gpu_memcpy_d2d(b.ptr, a.ptr, x.nbytes) == 0
+        assert gpu.gpu_memset(b.ptr + off, val, ln) == 0
+        want = x.copy()
+        want[off:off + ln] = val
+        assert (b.download(np.uint8, x.size) == want).all(), (off, ln)
+    # asynchronous copy lands by the stream sync (lm_adam.c:407-413,500)
+    host = np.zeros(x.size, np.uint8)
+    assert gpu.gpu_host_pin(host.ctypes.data, host.nbytes) == 0
+    assert gpu.gpu_host_pin(host.ctypes.data, host.nbytes) == 0
+    assert gpu.gpu_memcpy_d2h_async(host.ctypes.data, a.ptr, x.nbytes) == 0
+    assert gpu.gpu_stream_sync() == 0
+    assert (host == x).all()
+    gpu.gpu_host_forget(host.ctypes.data)
+    # argument checks as gpu_cuda.cu:2964-3029
+    assert gpu.gpu_memcpy_h2d(None, x.ctypes.data, 4) == -1
+    assert gpu.gpu_memcpy_d2h(x.ctypes.data, a.ptr, 0) == -1
+    assert gpu.gpu_memset(None, 0, 4) == -1
+    assert gpu.gpu_malloc(0) is None
+    hp = gpu.gpu_host_alloc(4096)
+    assert hp
+    gpu.gpu_host_free(hp)
+    gpu.gpu_device_sync()
+
+
+@pytest.mark.parametrize("n", [1, 3, 255, 4096, 4097, 65536 + 5, 3000017])
+def test_grad_sumsq(gpu, oracle, n):
+    rng = np.random.default_rng(n)
+    g = (rng.standard_normal(n) * 3e-2).astype(np.float32)
+    d = dev(gpu, g)
+    out = C.c_double(0)
+    assert gpu.gpu_grad_sumsq(d.ptr, n, C.byref(out)) == 0
+    want = oracle.sumsq(g)
+    assert abs(out.value - want) <= 1e-13 * want
+    first = out.value
+    for _ in range(3):                      # run-to-run deterministic
+        assert gpu.gpu_grad_sumsq(d.ptr, n, C.byref(out)) == 0 and out.value == first
+    # arguments (gpu_cuda.cu:8488-8489)
+    assert gpu.gpu_grad_sumsq(None, n, C.byref(out)) == -1
+    assert gpu.gpu_grad_sumsq(d.ptr, 0, C.byref(out)) == -1
+    assert gpu.gpu_grad_sumsq(d.ptr, n, None) == -1
+
+
+def test_grad_sumsq_unaligned_and_nonfinite(gpu, oracle):
+    rng = np.random.default_rng(77)
+    g = rng.standard_normal(20001).astype(np.float32)
+    d = dev(gpu, g)
+    out = C.c_double(0)
+    assert gpu.gpu_grad_sumsq(d.ptr + 4, 20000, C.byref(out)) == 0      # 4-byte aligned only
+    want = oracle.sumsq(g[1:])
+    assert abs(out.value - want) <= 1e-13 * want
+    for bad in (np.nan, np.inf):
+        g2 = g.copy()
+        g2[12345] = bad
+        d2 = dev(gpu, g2)
+        assert gpu.gpu_grad_sumsq(d2.ptr, g2.size, C.byref(out)) == 0
+        assert not math.isfinite(out.value)
+
+
+class FlatState:
+    """p/g/m/v/twin on the device + the same on the host for the oracle."""
+
+    def __init__(self, gpu, n, seed, twin=True):
+        rng = np.random.default_rng(seed)
+        self.gpu, self.n, self.rng = gpu, n, rng
+        self.p = (rng.standard_normal(n) * 0.02).astype(np.float32)
+        self.m = np.zeros(n, np.float32)
+        self.v = np.zeros(n, np.float32)
+        self.g = np.zeros(n, np.float32)
+        self.twin = np.zeros(n, np.uint16) if twin else None
+        self.dp, self.dm, self.dv = dev(gpu, self.p), dev(gpu, self.m), dev(gpu, self.v)
+        self.dg = dev(gpu, self.g)
+        self.dt = dev(gpu, np.zeros(n, np.uint16))
+
+    def new_grad(self, scale):
+        g = (self.rng.standard_normal(self.n) * scale).astype(np.float32)
+        self.g[:] = g
+        self.dg.upload(g)
+
+    def fetch(self):
+        f32 = np.float32
+        return (self.dp.download(f32, self.n), self.dm.download(f32, self.n),
+                self.dv.download(f32, self.n), self.dg.download(f32, self.n),
+                self.dt.download(np.uint16, self.n))
+
+
+@pytest.mark.parametrize("n,wd", [(1000003, 0.1), (4096 * 3, 0.0), (5, 0.1)])
+def test_flat_step_bit_exact_over_ten_steps(gpu, oracle, n, wd):
+    """gpu_adam_step_dev_bf16 with the grad_scale given: identical arithmetic -> identical bits."""
+    S = FlatState(gpu, n, seed=n)
+    O = oracle.Oracle(n, beta2=0.95, weight_decay=wd, threads=8)
+    gpu.gpu_set_compute_prec(1)
+    gpu.gpu_adam_set_weight_decay(wd)
+    for t in range(1, 11):
+        S.new_grad(1e-3 * (1 + (t % 4)))
+        lr = oracle.lr(3e-4, t - 1, 100, 1000, "cosine")
+        gs = 1.0 / (1 + t)
+        assert gpu.gpu_adam_step_dev_bf16(S.dp.ptr, S.dt.ptr, S.dg.ptr, S.dm.ptr, S.dv.ptr, n, lr,
+                                          0.9, 0.95, 1e-8, t, gs) == 0
+        O.step(S.p, S.g, S.m, S.v, lr, gs, twin=S.twin)
+        p, m, v, g, tw = S.fetch()
+        assert same_bits(p, S.p), t
+        assert same_bits(m, S.m) and same_bits(v, S.v), t
+        assert not g.any()                          # d_grad is zeroed by the step (gpu.h:125-127)
+        assert (tw == S.twin).all()
+        assert (tw == oracle.bf16_rne(p)).all()     # twin = RNE of the final p
+    gpu.gpu_set_compute_prec(0)
+    gpu.gpu_adam_set_weight_decay(0.0)
+
+
+def test_flat_step_without_bf16_precision_leaves_twins_alone(gpu, oracle):
+    n = 10000
+    S = FlatState(gpu, n, seed=3)
+    S.dt.upload(np.full(n, 0x1234, np.uint16))
+    gpu.gpu_set_compute_prec(0)                     # twins only when prec == BF16 (gpu_cuda.cu:8687,8704)
+    S.new_grad(1e-3)
+    assert gpu.gpu_adam_step_dev_bf16(S.dp.ptr, S.dt.ptr, S.dg.ptr, S.dm.ptr, S.dv.ptr, n, 1e-3,
+                                      0.9, 0.999, 1e-8, 1, 1.0) == 0
+    assert (S.dt.download(np.uint16, n) == 0x1234).all()
+    O = oracle.Oracle(n)
+    O.step(S.p, S.g, S.m, S.v, 1e-3)
+    assert same_bits(S.dp.download(np.float32, n), S.p)
+    # NULL twin pointer with BF16 precision is fine too
+    gpu.gpu_set_compute_prec(1)
+    S.new_grad(1e-3)
+    assert gpu.gpu_adam_step_dev_bf16(S.dp.ptr, None, S.dg.ptr, S.dm.ptr, S.dv.ptr, n, 1e-3,
+                                      0.9, 0.999, 1e-8, 2, 1.0) == 0
+    O.step(S.p, S.g, S.m, S.v, 1e-3)
+    assert same_bits(S.dp.download(np.float32, n), S.p)
+    gpu.gpu_set_compute_prec(0)
+
+
+def test_flat_step_unaligned_pointers(gpu, oracle):
+    """Pointers that are only 4-byte aligned take the element-wise path; same results."""
+    n = 9001
+    S = FlatState(gpu, n + 1, seed=21)
+    S.new_grad(1e-3)
+    gpu.gpu_set_compute_prec(1)
+    gpu.gpu_adam_set_weight_decay(0.1)
+    assert gpu.gpu_adam_step_dev_bf16(S.dp.ptr + 4, S.dt.ptr + 2, S.dg.ptr + 4, S.dm.ptr + 4,
+                                      S.dv.ptr + 4, n, 1e-3, 0.9, 0.95, 1e-8, 1, 0.5) == 0
+    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1)
+    p, g, m, v, tw = S.p[1:].copy(), S.g[1:].copy(), S.m[1:].copy(), S.v[1:].copy(), S.twin[1:].copy()
+    O.step(p, g, m, v, 1e-3, 0.5, twin=tw)
+    dp, dm, dv, dg, dt = S.fetch()
+    assert same_bits(dp[1:], p) and same_bits(dm[1:], m) and same_bits(dv[1:], v)
+    assert (dt[1:] == tw).all() and not dg[1:].any()
+    assert dp[0] == S.p[0] and dg[0] == S.g[0] and dt[0] == 0      # element before the range untouched
+    gpu.gpu_set_compute_prec(0)
+    gpu.gpu_adam_set_weight_decay(0.0)
+
+
+def test_flat_step_argument_checks(gpu):
+    """gpu_cuda.cu:8675-8682."""
+    S = FlatState(gpu, 64, seed=1)
+    ok = (S.dp.ptr, S.dt.ptr, S.dg.ptr, S.dm.ptr, S.dv.ptr)
+    f = gpu.gpu_adam_step_dev_bf16
+    assert f(None, ok[1], ok[2], ok[3], ok[4], 64, 1e-3, 0.9, 0.95, 1e-8, 1, 1.0) == -1
+    assert f(ok[0], ok[1], None, ok[3], ok[4], 64, 1e-3, 0.9, 0.95, 1e-8, 1, 1.0) == -1
+    assert f(ok[0], ok[1], ok[2], None, ok[4], 64, 1e-3, 0.9, 0.95, 1e-8, 1, 1.0) == -1
+    assert f(ok[0], ok[1], ok[2], ok[3], None, 64, 1e-3, 0.9, 0.95, 1e-8, 1, 1.0) == -1
+    assert f(*ok, 0, 1e-3, 0.9, 0.95, 1e-8, 1, 1.0) == -1
+    assert f(*ok, 64, 0.0, 0.9, 0.95, 1e-8, 1, 1.0) == -1
+    assert f(*ok, 64, 1e-3, 0.9, 0.95, 1e-8, 0, 1.0) == -1
+    assert f(*ok, 64, 1e-3, 1.0, 0.95, 1e-8, 1, 1.0) == -1         # 1 - beta1^t == 0
+    p = S.dp.download(np.float32, 64)
+    assert same_bits(p, S.p)                                        # nothing ran
+    gpu.gpu_adam_set_weight_decay(-3.0)                             # negatives clamp to 0
+
+
+def reference_device_flow(gpu, S, t, lr, grad_scale, clip, wd):
+    """The control flow of adam_step_gpu (lang/lm_adam.c:466-495) on the flat ABI."""
+    ss = C.c_double(0)
+    assert gpu.gpu_grad_sumsq(S.dg.ptr, S.n, C.byref(ss)) == 0
+    norm = math.sqrt(ss.value) * abs(grad_scale)
+    if not math.isfinite(norm):
+        assert gpu.gpu_memset(S.dg.ptr, 0, S.n * 4) == 0
+        return norm, True
+    if clip > 0 and norm > clip:
+        grad_scale *= clip / norm
+    gpu.gpu_adam_set_weight_decay(wd)
+    assert gpu.gpu_adam_step_dev_bf16(S.dp.ptr, S.dt.ptr, S.dg.ptr, S.dm.ptr, S.dv.ptr, S.n, lr,
+                                      0.9, 0.95, 1e-8, t, grad_scale) == 0
+    assert gpu.gpu_stream_sync() == 0
+    gpu.gpu_half_wt_invalidate(None)
+    return norm, False
+
+
+def test_unchanged_caller_flow_matches_cpu_path(gpu, oracle):
+    """What lang/lm_adam.c does with this backend vs its own host loop: BASELINE tolerances.
+    (The caller's device branch scales by clip/norm, its host loop by clip/(norm+1e-12).)"""
+    n = 300007
+    S = FlatState(gpu, n, seed=5)
+    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, threads=8)
+    gpu.gpu_set_compute_prec(1)
+    e0 = gpu.gpu_param_epoch()
+    clipped = 0
+    for t in range(1, 11):
+        S.new_grad(1e-3 * (1.0 if t % 2 else 4.0))      # sqrt(n)*1e-3 = 0.55 -> every other step clips
+        lr = oracle.lr(3e-4, t - 1, 100, 1000, "cosine")
+        norm, skipped = reference_device_flow(gpu, S, t, lr, 1.0, 1.0, 0.1)
+        O.step(S.p, S.g, S.m, S.v, lr, 1.0, twin=S.twin)
+        assert not skipped
+        assert abs(norm - O.o.last_grad_norm) <= TOL_NORM * O.o.last_grad_norm
+        clipped += O.o.last_clipped
+        p, m, v, g, tw = S.fetch()
+        assert rel_err(p, S.p) <= TOL_STATE and rel_err(m, S.m) <= TOL_STATE
+        assert rel_err(v, S.v) <= TOL_STATE
+        assert bf16_ulp_diff(tw, S.twin) <= 1 and not g.any()
+    assert clipped == 5 and gpu.gpu_param_epoch() == e0 + 10
+    gpu.gpu_set_compute_prec(0)
+    gpu.gpu_adam_set_weight_decay(0.0)
+
+
+def test_unchanged_caller_flow_skips_nonfinite(gpu):
+    n = 5000
+    S = FlatState(gpu, n, seed=6)
+    S.new_grad(1e-3)
+    g = S.g.copy()
+    g[77] = np.nan
+    S.dg.upload(g)
+    norm, skipped = reference_device_flow(gpu, S, 1, 1e-3, 1.0, 1.0, 0.1)
+    assert skipped and math.isnan(norm)
+    p, m, v, gg, _tw = S.fetch()
+    assert same_bits(p, S.p) and not m.any() and not v.any() and not gg.any()
+
+
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+def test_golden_vectors_through_flat_abi(gpu, name):
+    """The reference's own outputs (written by its compiled host loop) vs this backend."""
+    G = load_golden(name)
+    n = G["p0"].size
+    S = FlatState(gpu, n, seed=0)
+    S.dp.upload(G["p0"])
+    clip, wd, gs0 = float(G["clip"]), float(G["wd"]), float(G["grad_scale"])
+    gpu.gpu_set_compute_prec(1)
+    for s in range(G["grads"].shape[0]):
+        S.dg.upload(G["grads"][s])
+        if clip > 0:
+            reference_device_flow(gpu, S, s + 1, float(G["lr"][s]), gs0, clip, wd)
+        else:
+            gpu.gpu_adam_set_weight_decay(wd)
+            assert gpu.gpu_adam_step_dev_bf16(S.dp.ptr, S.dt.ptr, S.dg.ptr, S.dm.ptr, S.dv.ptr, n,
+                                              float(G["lr"][s]), float(G["beta1"]),
+                                              float(G["beta2"]), float(G["eps"]), s + 1, gs0) == 0
+        p, m, v, g, _tw = S.fetch()
+        if clip > 0:
+            assert rel_err(p, G["p"][s]) <= TOL_STATE and rel_err(m, G["m"][s]) <= TOL_STATE
+            assert rel_err(v, G["v"][s]) <= TOL_STATE
+        else:
+            assert same_bits(p, G["p"][s]) and same_bits(m, G["m"][s]) and same_bits(v, G["v"][s])
+        assert not g.any()
+    gpu.gpu_set_compute_prec(0)
+    gpu.gpu_adam_set_weight_decay(0.0)
+
+
+def test_seed_bf16_flat(gpu, oracle):
+    for n in (1, 7, 4096, 100003):
+        x = (np.random.default_rng(n).standard_normal(n) * 0.02).astype(np.float32)
+        d = dev(gpu, x)
+        o = dev(gpu, np.zeros(n, np.uint16))
+        gpu.gpu_adam_set_bf16_flat(o.ptr, d.ptr, n)
+        assert gpu.gpu_adam_seed_bf16_flat(o.ptr, d.ptr, n) == 0
+        assert (o.download(np.uint16, n) == oracle.bf16_rne(x)).all()
+        gpu.gpu_adam_set_bf16_flat(None, None, 0)
+    assert gpu.gpu_adam_seed_bf16_flat(None, None, 5) == -1
