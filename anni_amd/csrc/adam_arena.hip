@@ -26,10 +26,13 @@ struct anni_adam_priv {
 	double			*d_partials;
 	StepState		*d_state;
 	StepState		*h_state;	/* page-locked */
-	void			*own_grad;	/* the arena's gradient flat (NULL when external) */
+	char			*grad_slots;	/* the arena's gradient flats (NULL when external) */
+	size_t			grad_slot_bytes;	/* distance between consecutive slots */
+	int			n_grad_slots;
+	int			spread;		/* 1: every flat in its own region of device memory */
+	double			probe_gbps;	/* update throughput measured at creation (0: not measured) */
 	std::vector<int64_t>	offsets;
 	std::vector<uint32_t>	flags;
-	bool			any_decay_off;
 };
 
 static size_t elem_bytes(int type)
@@ -37,9 +40,185 @@ static size_t elem_bytes(int type)
 	return type == ANNI_F32 ? 4 : type == ANNI_BF16 ? 2 : 1;
 }
 
+/* Size of one region of device memory (see the layout note in anni_adam_create); ANNI_REGION_GIB overrides. */
+static size_t region_bytes(void)
+{
+	static size_t r;
+
+	if (!r) {
+		const char *e = getenv("ANNI_REGION_GIB");
+		long g = e ? atol(e) : 16;
+
+		if (g < 1 || g > 64)
+			g = 16;
+		r = (size_t)g << 30;
+	}
+	return r;
+}
+
 static size_t round_up(size_t x, size_t a)
 {
 	return (x + a - 1) / a * a;
+}
+
+/* Byte sizes of the flats of one arena. */
+struct Sizes {
+	int64_t	n;
+	int	n_tensors;
+	int64_t	n_tiles;
+	int	n_slots;
+	size_t	p_bytes;
+	size_t	mv_bytes;
+	size_t	tw_bytes;
+	size_t	g_bytes;	/* one gradient slot, rounded up to 2 MiB */
+};
+
+/* One device allocation with the flats laid out in it. */
+struct Placement {
+	void	*arena;
+	size_t	total;
+	size_t	off_p, off_m, off_v, off_twin, off_g, off_gscale, off_segs, off_tiles, off_part,
+		off_state;
+	int	spread;
+	double	gbps;		/* what the probe measured (0: not probed) */
+};
+
+/*
+** Layout.  On MI355X a kernel that streams several arrays at once runs about 20 %
+** faster when the arrays lie in different 16 GiB regions of device memory than when two
+** of them share one (measured: 6.2 against 5.1 TB/s for this update; a kernel with a
+** single stream does not care).  SPREAD therefore puts p, m, v and the twins one region
+** apart and the gradient slots behind them, all inside ONE allocation whose size is a
+** whole number of regions, so same-index elements of any two flats are a whole number
+** of regions apart.  The holes are reserved with it.  COMPACT packs the flats at 2 MiB
+** boundaries.
+*/
+static bool place(const Sizes &z, bool spread, Placement *pl)
+{
+	const size_t big = (size_t)2 << 20;
+	const size_t stride = spread ? round_up(z.p_bytes, region_bytes()) : 0;
+
+	memset(pl, 0, sizeof(*pl));
+	pl->off_p = 0;
+	pl->off_m = spread ? stride : round_up(pl->off_p + z.p_bytes, big);
+	pl->off_v = spread ? 2 * stride : round_up(pl->off_m + z.mv_bytes, big);
+	pl->off_twin = spread ? 3 * stride : round_up(pl->off_v + z.mv_bytes, big);
+	pl->off_g = spread ? 4 * stride : round_up(pl->off_twin + z.tw_bytes, big);
+	pl->off_gscale = round_up(pl->off_g + (size_t)z.n_slots * z.g_bytes, big);
+	pl->off_segs = pl->off_gscale + round_up((size_t)z.n_tensors * sizeof(float), 256);
+	pl->off_tiles = pl->off_segs + round_up((size_t)z.n_tensors * sizeof(Seg), 256);
+	pl->off_part = pl->off_tiles + round_up((size_t)z.n_tiles * sizeof(int32_t), 256);
+	pl->off_state = pl->off_part + round_up((size_t)kMaxPartials * sizeof(double), 256);
+	pl->total = pl->off_state + 256;
+	if (spread)
+		pl->total = round_up(pl->total, region_bytes());
+	pl->spread = spread ? 1 : 0;
+	if (hipMalloc(&pl->arena, pl->total) != hipSuccess) {
+		(void)hipGetLastError();
+		pl->arena = nullptr;
+		return false;
+	}
+	return true;
+}
+
+/* Points the handle at a placement. */
+static void adopt(anni_adam *opt, const Sizes &z, const Placement &pl)
+{
+	anni_adam_priv *pv = opt->priv;
+	char *base = (char *)pl.arena;
+
+	pv->arena = pl.arena;
+	pv->arena_bytes = pl.total;
+	pv->spread = pl.spread;
+	pv->probe_gbps = pl.gbps;
+	opt->d_param = (float *)(base + pl.off_p);
+	opt->d_m = base + pl.off_m;
+	opt->d_v = base + pl.off_v;
+	opt->d_param_bf16 = z.tw_bytes ? base + pl.off_twin : nullptr;
+	pv->grad_slots = z.n_slots ? base + pl.off_g : nullptr;
+	pv->grad_slot_bytes = z.g_bytes;
+	pv->n_grad_slots = z.n_slots;
+	opt->d_grad = pv->grad_slots;
+	opt->d_gscale = (float *)(base + pl.off_gscale);
+	pv->d_segs = (Seg *)(base + pl.off_segs);
+	pv->d_tile_seg = (int32_t *)(base + pl.off_tiles);
+	pv->d_partials = (double *)(base + pl.off_part);
+	pv->d_state = (StepState *)(base + pl.off_state);
+}
+
+/* State starts at zero (slots are calloc'ed, lm_adam.c:92); tables are uploaded; all on the stream. */
+static bool init_contents(anni_adam *opt, const Sizes &z, const Placement &pl,
+	const std::vector<Seg> &segs, const std::vector<int32_t> &tile_seg)
+{
+	char *base = (char *)pl.arena;
+	hipStream_t st = compute_stream();
+	std::vector<float> ones((size_t)z.n_tensors, 1.0f);
+
+	return launch_fill_bytes(st, base + pl.off_p, 0, z.p_bytes) == 0
+	    && launch_fill_bytes(st, base + pl.off_m, 0, z.mv_bytes) == 0
+	    && launch_fill_bytes(st, base + pl.off_v, 0, z.mv_bytes) == 0
+	    && (!z.tw_bytes || launch_fill_bytes(st, base + pl.off_twin, 0, z.tw_bytes) == 0)
+	    && (!z.n_slots || launch_fill_bytes(st, base + pl.off_g, 0,
+	    (size_t)z.n_slots * z.g_bytes) == 0)
+	    && launch_fill_bytes(st, base + pl.off_part, 0, pl.off_state + 256 - pl.off_part) == 0
+	    && hip_ok(hipMemcpyAsync(opt->d_gscale, ones.data(), (size_t)z.n_tensors * sizeof(float),
+	    hipMemcpyHostToDevice, st), "gscale")
+	    && hip_ok(hipMemcpyAsync(opt->priv->d_segs, segs.data(), (size_t)z.n_tensors * sizeof(Seg),
+	    hipMemcpyHostToDevice, st), "segs")
+	    && hip_ok(hipMemcpyAsync(opt->priv->d_tile_seg, tile_seg.data(),
+	    (size_t)z.n_tiles * sizeof(int32_t), hipMemcpyHostToDevice, st), "tiles")
+	    && hip_ok(hipStreamSynchronize(st), "arena init");
+}
+
+static void describe(const anni_adam *opt, Flat *f);
+
+/*
+** Throughput of the update on this placement, in GB/s of algorithmic traffic.  Run on
+** the all-zero state it leaves every flat as it is (0 stays 0 under the update).
+*/
+static double probe(const anni_adam *opt)
+{
+	hipStream_t st = compute_stream();
+	hipEvent_t e0, e1;
+	StepConsts c;
+	NormIn norm;
+	Flat f;
+	float ms = 0.0f;
+	const double bytes = (double)opt->n * (8.0 + 2.0 * elem_bytes(opt->cfg.grad_type)
+	    + 4.0 * elem_bytes(opt->cfg.moment_type) + (opt->d_param_bf16 ? 2.0 : 0.0));
+
+	if (!opt->d_grad)
+		return 0.0;
+	memset(&c, 0, sizeof(c));
+	c.beta1 = 0.9;
+	c.omb1 = 1.0 - 0.9;
+	c.beta2 = 0.95;
+	c.omb2 = 1.0 - 0.95;
+	c.eps = 1e-8;
+	c.bc1 = c.omb1;
+	c.bc2 = c.omb2;
+	c.lr = 1e-3;
+	memset(&norm, 0, sizeof(norm));
+	describe(opt, &f);
+	if (hipEventCreate(&e0) != hipSuccess)
+		return 0.0;
+	if (hipEventCreate(&e1) != hipSuccess) {
+		(void)hipEventDestroy(e0);
+		return 0.0;
+	}
+	if (launch_update(st, f, c, 1.0, norm) == 0) {
+		(void)hipEventRecord(e0, st);
+		(void)launch_update(st, f, c, 1.0, norm);
+		(void)launch_update(st, f, c, 1.0, norm);
+		(void)hipEventRecord(e1, st);
+		if (hipStreamSynchronize(st) != hipSuccess
+		    || hipEventElapsedTime(&ms, e0, e1) != hipSuccess)
+			ms = 0.0f;
+	}
+	(void)hipGetLastError();
+	(void)hipEventDestroy(e0);
+	(void)hipEventDestroy(e1);
+	return ms > 0.0f ? 2.0 * bytes / (ms * 1e-3) / 1e9 : 0.0;
 }
 
 extern "C" {
@@ -48,20 +227,26 @@ anni_adam *anni_adam_create(const anni_tensor *tensors, int n_tensors,
 	const anni_adam_config *cfg)
 {
 	const size_t big = (size_t)2 << 20;	/* each flat starts on a 2 MiB boundary */
+	/* A spread placement is tried again (up to kTries) while the probe stays below kGoodGBps. */
+	const int kTries = 3;
+	const double kGoodGBps = 5600.0;
 	anni_adam *opt;
 	anni_adam_priv *pv;
-	int64_t n = 0;
-	size_t off_p, off_m, off_v, off_twin, off_g, off_gscale, off_segs, off_tiles, off_part,
-	    off_state, total;
-	int64_t n_tiles;
+	Sizes z;
 	std::vector<Seg> segs;
 	std::vector<int32_t> tile_seg;
-	std::vector<float> ones;
+	std::vector<Placement> tried;
+	Placement pl;
+	int64_t n = 0;
+	bool want_spread;
+	bool ok = false;
 
 	if (!tensors || n_tensors <= 0 || !cfg || !device_ready())
 		return nullptr;
 	if (cfg->grad_type < ANNI_F32 || cfg->grad_type > ANNI_FP8_E4M3
-	    || (cfg->moment_type != ANNI_F32 && cfg->moment_type != ANNI_BF16))
+	    || (cfg->moment_type != ANNI_F32 && cfg->moment_type != ANNI_BF16)
+	    || cfg->grad_slots < 0 || cfg->grad_slots > 4096
+	    || cfg->layout < ANNI_LAYOUT_AUTO || cfg->layout > ANNI_LAYOUT_SPREAD)
 		return nullptr;
 	for (int i = 0; i < n_tensors; i++) {
 		if (tensors[i].n < 0)
@@ -103,74 +288,91 @@ anni_adam *anni_adam_create(const anni_tensor *tensors, int n_tensors,
 		}
 	}
 	/* Launch table: the tensor that holds the first element of each tile. */
-	n_tiles = (n + kTile - 1) / kTile;
-	tile_seg.resize((size_t)n_tiles);
+	z.n = n;
+	z.n_tensors = n_tensors;
+	z.n_tiles = (n + kTile - 1) / kTile;
+	z.n_slots = cfg->grad_slots;
+	z.p_bytes = (size_t)n * 4;
+	z.mv_bytes = (size_t)n * elem_bytes(cfg->moment_type);
+	z.tw_bytes = cfg->twins ? (size_t)n * 2 : 0;
+	z.g_bytes = round_up((size_t)n * elem_bytes(cfg->grad_type), big);
+	tile_seg.resize((size_t)z.n_tiles);
 	{
 		int s = 0;
 
-		for (int64_t k = 0; k < n_tiles; k++) {
+		for (int64_t k = 0; k < z.n_tiles; k++) {
 			while (segs[(size_t)s].end <= k * kTile)
 				s++;
 			tile_seg[(size_t)k] = s;
 		}
 	}
-
-	off_p = 0;
-	off_m = round_up(off_p + (size_t)n * 4, big);
-	off_v = round_up(off_m + (size_t)n * elem_bytes(cfg->moment_type), big);
-	off_twin = round_up(off_v + (size_t)n * elem_bytes(cfg->moment_type), big);
-	off_g = round_up(off_twin + (cfg->twins ? (size_t)n * 2 : 0), big);
-	off_gscale = round_up(off_g + (cfg->own_grad ? (size_t)n * elem_bytes(cfg->grad_type) : 0),
-	    big);
-	off_segs = round_up(off_gscale + (size_t)n_tensors * sizeof(float), 256);
-	off_tiles = round_up(off_segs + (size_t)n_tensors * sizeof(Seg), 256);
-	off_part = round_up(off_tiles + (size_t)n_tiles * sizeof(int32_t), 256);
-	off_state = round_up(off_part + (size_t)kMaxPartials * sizeof(double), 256);
-	total = off_state + 256;
-
-	if (!hip_ok(hipMalloc(&pv->arena, total), "arena hipMalloc")
-	    || !hip_ok(hipHostMalloc((void **)&pv->h_state, sizeof(StepState),
-	    hipHostMallocDefault), "arena hipHostMalloc")) {
+	if (!hip_ok(hipHostMalloc((void **)&pv->h_state, sizeof(StepState), hipHostMallocDefault),
+	    "arena hipHostMalloc")) {
 		(void)hipGetLastError();
 		anni_adam_free(&opt);
 		return nullptr;
 	}
-	pv->arena_bytes = total;
-	{
-		char *base = (char *)pv->arena;
-		hipStream_t st = compute_stream();
+	memset(pv->h_state, 0, sizeof(StepState));
 
-		opt->d_param = (float *)(base + off_p);
-		opt->d_m = base + off_m;
-		opt->d_v = base + off_v;
-		opt->d_param_bf16 = cfg->twins ? base + off_twin : nullptr;
-		pv->own_grad = cfg->own_grad ? base + off_g : nullptr;
-		opt->d_grad = pv->own_grad;
-		opt->d_gscale = (float *)(base + off_gscale);
-		pv->d_segs = (Seg *)(base + off_segs);
-		pv->d_tile_seg = (int32_t *)(base + off_tiles);
-		pv->d_partials = (double *)(base + off_part);
-		pv->d_state = (StepState *)(base + off_state);
+	/*
+	** AUTO spreads flats of 256 MiB and more (smaller ones are not bandwidth critical),
+	** and only while the spread arena takes less than half of what is free.
+	*/
+	want_spread = cfg->layout == ANNI_LAYOUT_SPREAD;
+	if (cfg->layout == ANNI_LAYOUT_AUTO && z.p_bytes >= ((size_t)256 << 20)) {
+		size_t free_b = 0, total_b = 0;
+		const size_t need = round_up(4 * round_up(z.p_bytes, region_bytes())
+		    + (size_t)z.n_slots * z.g_bytes + ((size_t)64 << 20), region_bytes());
 
-		ones.assign((size_t)n_tensors, 1.0f);
-		/* State starts at zero (slots are calloc'ed, lm_adam.c:92); the fills run on the stream. */
-		if (launch_fill_bytes(st, base + off_p, 0, off_twin) != 0
-		    || (cfg->twins && launch_fill_bytes(st, base + off_twin, 0, (size_t)n * 2) != 0)
-		    || (cfg->own_grad && launch_fill_bytes(st, base + off_g, 0,
-		    (size_t)n * elem_bytes(cfg->grad_type)) != 0)
-		    || launch_fill_bytes(st, base + off_part, 0, total - off_part) != 0
-		    || !hip_ok(hipMemcpyAsync(opt->d_gscale, ones.data(),
-		    (size_t)n_tensors * sizeof(float), hipMemcpyHostToDevice, st), "gscale")
-		    || !hip_ok(hipMemcpyAsync(pv->d_segs, segs.data(),
-		    (size_t)n_tensors * sizeof(Seg), hipMemcpyHostToDevice, st), "segs")
-		    || !hip_ok(hipMemcpyAsync(pv->d_tile_seg, tile_seg.data(),
-		    (size_t)n_tiles * sizeof(int32_t), hipMemcpyHostToDevice, st), "tiles")
-		    || !hip_ok(hipStreamSynchronize(st), "arena init")) {
-			anni_adam_free(&opt);
-			return nullptr;
+		if (hipMemGetInfo(&free_b, &total_b) == hipSuccess && need <= free_b / 2)
+			want_spread = true;
+		(void)hipGetLastError();
+	}
+	if (want_spread) {
+		/*
+		** Where a placement lands physically is the driver's choice and it shows in the
+		** throughput, so a slow one is kept aside (which makes the next one land
+		** elsewhere) and the fastest of a few is used.  Only with gradient slots to run on.
+		*/
+		const bool audition = z.n_slots > 0 && z.p_bytes >= ((size_t)256 << 20);
+
+		for (int k = 0; k < kTries; k++) {
+			if (!place(z, true, &pl))
+				break;
+			adopt(opt, z, pl);
+			if (!init_contents(opt, z, pl, segs, tile_seg)) {
+				(void)hipFree(pl.arena);
+				break;
+			}
+			pl.gbps = audition ? probe(opt) : 0.0;
+			tried.push_back(pl);
+			if (!audition || pl.gbps >= kGoodGBps)
+				break;
+		}
+		if (!tried.empty()) {
+			size_t best = 0;
+
+			for (size_t k = 1; k < tried.size(); k++)
+				if (tried[k].gbps > tried[best].gbps)
+					best = k;
+			for (size_t k = 0; k < tried.size(); k++)
+				if (k != best)
+					(void)hip_ok(hipFree(tried[k].arena), "arena hipFree");
+			adopt(opt, z, tried[best]);
+			ok = true;
 		}
 	}
-	memset(pv->h_state, 0, sizeof(StepState));
+	if (!ok && cfg->layout != ANNI_LAYOUT_SPREAD) {
+		if (place(z, false, &pl)) {
+			adopt(opt, z, pl);
+			ok = init_contents(opt, z, pl, segs, tile_seg);
+		}
+	}
+	if (!ok) {
+		(void)hip_ok(hipErrorOutOfMemory, "arena hipMalloc");
+		anni_adam_free(&opt);
+		return nullptr;
+	}
 	return opt;
 }
 
@@ -205,8 +407,25 @@ int anni_adam_bind_grad(anni_adam *opt, void *d_grad)
 {
 	if (!opt || !opt->priv)
 		return -1;
-	opt->d_grad = d_grad ? d_grad : opt->priv->own_grad;
+	opt->d_grad = d_grad ? d_grad : (void *)opt->priv->grad_slots;
 	return opt->d_grad ? 0 : -1;
+}
+
+void *anni_adam_grad_slot(const anni_adam *opt, int k)
+{
+	if (!opt || !opt->priv || k < 0 || k >= opt->priv->n_grad_slots)
+		return nullptr;
+	return opt->priv->grad_slots + (size_t)k * opt->priv->grad_slot_bytes;
+}
+
+int anni_adam_is_spread(const anni_adam *opt)
+{
+	return opt && opt->priv ? opt->priv->spread : 0;
+}
+
+double anni_adam_probe_gbps(const anni_adam *opt)
+{
+	return opt && opt->priv ? opt->priv->probe_gbps : 0.0;
 }
 
 int anni_adam_seed_twins(anni_adam *opt)

@@ -11,6 +11,7 @@ SO_PATH = os.path.join(HERE, "libanni_gpu_hip.so")
 
 F32, BF16, FP8_E4M3 = 0, 1, 2
 T_DECAY, T_TWIN = 1, 2
+LAYOUT_AUTO, LAYOUT_COMPACT, LAYOUT_SPREAD = 0, 1, 2
 GPU_PREC_FP32, GPU_PREC_BF16 = 0, 1
 
 
@@ -26,7 +27,7 @@ class Tensor(C.Structure):
 class Config(C.Structure):
     """anni_adam_config."""
     _fields_ = [("grad_type", C.c_int), ("moment_type", C.c_int), ("twins", C.c_int),
-                ("skip_nonfinite", C.c_int), ("own_grad", C.c_int)]
+                ("skip_nonfinite", C.c_int), ("grad_slots", C.c_int), ("layout", C.c_int)]
 
 
 class Adam(C.Structure):
@@ -77,6 +78,9 @@ _PROTOS = {
     "anni_adam_create": (C.POINTER(Adam), [C.POINTER(Tensor), C.c_int, C.POINTER(Config)]),
     "anni_adam_free": (None, [C.POINTER(C.POINTER(Adam))]),
     "anni_adam_tensor_offset": (C.c_int64, [C.POINTER(Adam), C.c_int]),
+    "anni_adam_grad_slot": (C.c_void_p, [C.POINTER(Adam), C.c_int]),
+    "anni_adam_is_spread": (C.c_int, [C.POINTER(Adam)]),
+    "anni_adam_probe_gbps": (C.c_double, [C.POINTER(Adam)]),
     "anni_adam_bind_grad": (C.c_int, [C.POINTER(Adam), C.c_void_p]),
     "anni_adam_seed_twins": (C.c_int, [C.POINTER(Adam)]),
     "anni_adam_zero_grad": (C.c_int, [C.POINTER(Adam)]),

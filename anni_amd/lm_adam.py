@@ -65,13 +65,14 @@ class LmAdam:
     """lm_adam over a list of tensors ((n, flags) pairs or (name, n, flags) triples)."""
 
     def __init__(self, tensors, grad_type=_l.F32, moment_type=_l.F32, twins=True,
-                 skip_nonfinite=False, own_grad=True, beta1=0.9, beta2=0.999, eps=1e-8,
+                 skip_nonfinite=False, grad_slots=1, layout=_l.LAYOUT_AUTO, beta1=0.9, beta2=0.999, eps=1e-8,
                  weight_decay=0.0, grad_clip=0.0):
         self.L = _l.require_gpu()
         rows = [(t[-2], t[-1]) for t in tensors]
         self.names = [t[0] if len(t) == 3 else "t%d" % i for i, t in enumerate(tensors)]
         arr = (_l.Tensor * len(rows))(*[_l.Tensor(int(n), int(f)) for n, f in rows])
-        cfg = _l.Config(grad_type, moment_type, int(twins), int(skip_nonfinite), int(own_grad))
+        cfg = _l.Config(grad_type, moment_type, int(twins), int(skip_nonfinite), int(grad_slots),
+                         int(layout))
         self.h = self.L.anni_adam_create(arr, len(rows), C.byref(cfg))
         if not self.h:
             raise RuntimeError("anni_adam_create failed: %s"
@@ -119,6 +120,17 @@ class LmAdam:
         if self.L.anni_adam_sync_stats(self.h) != 0:
             raise RuntimeError("anni_adam_sync_stats failed")
         return self.o
+
+    def grad_slot(self, k):
+        return self.L.anni_adam_grad_slot(self.h, k)
+
+    @property
+    def spread(self):
+        return bool(self.L.anni_adam_is_spread(self.h))
+
+    @property
+    def probe_gbps(self):
+        return self.L.anni_adam_probe_gbps(self.h)
 
     def bind_grad(self, ptr):
         if self.L.anni_adam_bind_grad(self.h, ptr) != 0:

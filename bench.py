@@ -4,7 +4,7 @@
 A "step" is one pass of the optimizer over the whole parameter set of the named workload:
 the global sum of squares of the gradients (clip norm) and the fused update.  Inputs are
 synthetic and already resident in HBM when the timed region starts: parameters ~N(0, 0.02),
-zero moments, and one fresh gradient flat ~N(0, 1e-3) per step (a ring of steps+warmup flats,
+zero moments, and one fresh gradient flat ~N(0, 1e-3) per step (steps+warmup gradient slots of the arena,
 generated on the device), scaled so that about half the steps clip.  The learning rate follows
 a 100-step warmup + cosine schedule.
 
@@ -41,28 +41,32 @@ STORAGE = {"185m": "f32 p/g/m/v + bf16 twin", "555m": "f32 p/g/m/v + bf16 twin",
            "1p4b-fp8": "f32 p/m/v, fp8-e4m3 g with per-tensor scale + bf16 twin"}
 
 
-def make_grad_ring(L, opt, tensors, count, grad_type, seed):
-    """count gradient flats on the device, each ~N(0, 1e-3) in the workload's storage type."""
+def fill_grad_slots(L, opt, tensors, count, grad_type, seed):
+    """Fills the arena's `count` gradient slots, each ~N(0, 1e-3) in the workload's storage type.
+    Returns the slot pointers and, for fp8, one per-tensor scale array per slot."""
     from anni_amd.lm_adam import DeviceBuffer
     n = opt.n
-    ring, scales = [], []
+    ptrs, scales = [], []
     stage = DeviceBuffer(n * 4) if grad_type != 0 else None
     for k in range(count):
-        buf = DeviceBuffer(n * ELEM[grad_type])
-        dst = buf.ptr if grad_type == 0 else stage.ptr
+        slot = opt.grad_slot(k)
+        assert slot
+        dst = slot if grad_type == 0 else stage.ptr
         assert L.anni_fill_normal_f32(dst, n, seed, 1000 + k, 0.0, 1e-3) == 0
         sc = None
         if grad_type == 1:
-            assert L.anni_f32_to_bf16(buf.ptr, stage.ptr, n) == 0
+            assert L.anni_f32_to_bf16(slot, stage.ptr, n) == 0
         elif grad_type == 2:
             sc = DeviceBuffer(len(tensors) * 4)
             for i, (off, cnt) in enumerate(zip(opt.offsets, opt.sizes)):
-                assert L.anni_fp8_quantize(buf.ptr + off, sc.ptr + 4 * i, stage.ptr + 4 * off,
+                assert L.anni_fp8_quantize(slot + off, sc.ptr + 4 * i, stage.ptr + 4 * off,
                                            cnt) == 0
         assert L.gpu_stream_sync() == 0
-        ring.append(buf)
+        ptrs.append(slot)
         scales.append(sc)
-    return ring, scales
+    if stage is not None:
+        stage.free()
+    return ptrs, scales
 
 
 def cpu_baselines(size_name, norm_bpp, upd_bpp, budget_s):
@@ -154,6 +158,8 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="555m", choices=sorted(WORKLOADS))
+    ap.add_argument("--layout", default="auto", choices=["auto", "compact", "spread"],
+                    help="arena layout (spread: every flat in its own 16 GiB region)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds for the CPU legs")
     a = ap.parse_args()
@@ -169,13 +175,14 @@ def main():
 
     size, gt, mt, norm_bpp, upd_bpp = WORKLOADS[a.workload]
     tensors = layout.tensors(size)
+    total = a.steps + a.warmup
     opt = LmAdam(tensors, grad_type=gt, moment_type=mt, twins=True, skip_nonfinite=True,
-                 own_grad=False, beta2=0.95, weight_decay=0.1, grad_clip=1.0)
+                 grad_slots=total, layout={"auto": 0, "compact": 1, "spread": 2}[a.layout],
+                 beta2=0.95, weight_decay=0.1, grad_clip=1.0)
     n = opt.n
     assert L.anni_fill_normal_f32(opt.o.d_param, n, 20260101, 1, 0.0, 0.02) == 0
     opt.seed_twins()
-    total = a.steps + a.warmup
-    ring, scales = make_grad_ring(L, opt, tensors, total, gt, 20260101)
+    ring, scales = fill_grad_slots(L, opt, tensors, total, gt, 20260101)
 
     # per-step inputs: warmup(100)+cosine lr at schedule steps 0.., grad scale straddling the clip
     from anni_amd import lm_adam
@@ -184,7 +191,7 @@ def main():
     gss = [unit * (1.7 if s % 2 else 0.6) for s in range(total)]
 
     def run(first, count, per_kernel):
-        ptrs = (C.c_void_p * count)(*[ring[first + i].ptr for i in range(count)])
+        ptrs = (C.c_void_p * count)(*[ring[first + i] for i in range(count)])
         lr = (C.c_double * count)(*lrs[first:first + count])
         gs = (C.c_double * count)(*gss[first:first + count])
         ms, ms_a, ms_b = C.c_float(0), C.c_float(0), C.c_float(0)
@@ -233,6 +240,8 @@ def main():
         "config": {"workload": a.workload, "storage": STORAGE[a.workload], "params": n, "tensors": len(tensors),
                    "bytes_per_param": bpp, "clip": 1.0, "weight_decay": 0.1, "beta2": 0.95,
                    "lr": "3e-4 warmup100+cosine", "twins": "bf16 RNE on matrices",
+                   "layout": "spread" if opt.spread else "compact",
+                   "placement_probe_GBps": round(opt.probe_gbps, 1),
                    "launches_per_step": 2},
         "params_per_s": round(n / (ms_step * 1e-3), 1),
         "pct_of_hbm_peak": round(100.0 * step_gbps / HBM_PEAK_GBPS, 2),

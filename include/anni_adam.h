@@ -37,6 +37,19 @@ extern "C" {
 #define ANNI_BF16	1	/* upper 16 bits of an IEEE float */
 #define ANNI_FP8_E4M3	2	/* OCP E4M3: bias 7, max 448, S.1111.111 = NaN, no infinities */
 
+/*
+** Arena layouts.  SPREAD puts every flat into its own 16 GiB region of device memory
+** (one allocation, holes included), which is what lets a kernel that streams all of
+** them at once reach full HBM speed on MI355X; COMPACT packs them.  AUTO spreads when
+** the parameter flat is at least 256 MiB and the spread arena takes less than half of
+** the free device memory.  Where a spread arena lands physically is the driver's choice
+** and shows in the throughput: creation times the update on a few placements and keeps
+** the fastest (only when the arena owns gradient slots to run on).
+*/
+#define ANNI_LAYOUT_AUTO	0
+#define ANNI_LAYOUT_COMPACT	1
+#define ANNI_LAYOUT_SPREAD	2
+
 /* Tensor flags. */
 #define ANNI_T_DECAY	1u	/* decoupled weight decay applies (BASELINE: matrices only) */
 #define ANNI_T_TWIN	2u	/* the bf16 twin of this tensor is written */
@@ -52,7 +65,8 @@ typedef struct anni_adam_config {
 	int	moment_type;	/* ANNI_F32 / ANNI_BF16 (computed in double, rounded f32 then bf16 on store) */
 	int	twins;		/* 1: allocate the bf16 twin flat */
 	int	skip_nonfinite;	/* 1: a non-finite gradient norm skips the update (lm_adam.c:474-483) */
-	int	own_grad;	/* 1: the arena allocates the gradient flat; 0: bind one with anni_adam_bind_grad */
+	int	grad_slots;	/* gradient flats the arena allocates (slot 0 starts bound); 0: bind one with anni_adam_bind_grad */
+	int	layout;		/* ANNI_LAYOUT_AUTO / _COMPACT / _SPREAD */
 } anni_adam_config;
 
 struct anni_adam_priv;
@@ -72,7 +86,7 @@ typedef struct anni_adam {
 	int	last_skipped;
 	int	last_clipped;
 	anni_adam_config cfg;
-	/* the device arena: one allocation, each flat 2 MiB aligned */
+	/* the device arena: one allocation, each flat 2 MiB aligned (see ANNI_LAYOUT_*) */
 	float	*d_param;
 	void	*d_param_bf16;
 	void	*d_grad;
@@ -85,7 +99,7 @@ typedef struct anni_adam {
 /*
 ** Counterpart of lm_adam_create + gpu_buffers_init (lm_adam.c:79-139,217-311):
 ** registers the tensors in order at packed offsets, allocates the arena (p, m,
-** v zeroed; gradients zeroed when own_grad), builds the launch table.
+** v zeroed; gradient slots zeroed), builds the launch table.
 ** NULL on failure.
 */
 anni_adam	*anni_adam_create(const anni_tensor *tensors, int n_tensors,
@@ -94,7 +108,12 @@ anni_adam	*anni_adam_create(const anni_tensor *tensors, int n_tensors,
 void	anni_adam_free(anni_adam **opt);
 /* Element offset of tensor i in every flat. */
 int64_t	anni_adam_tensor_offset(const anni_adam *opt, int i);
-/* Use an external gradient flat (n elements of grad_type, e.g. written by backward). */
+/* Gradient slot k of the arena (k < cfg.grad_slots), else NULL; 1 when the layout came out SPREAD. */
+void	*anni_adam_grad_slot(const anni_adam *opt, int k);
+int	anni_adam_is_spread(const anni_adam *opt);
+/* GB/s of algorithmic traffic the update reached on this placement when the arena was created (0: not measured). */
+double	anni_adam_probe_gbps(const anni_adam *opt);
+/* Use another gradient flat: a slot of the arena or an external one (n elements of grad_type); NULL = slot 0. */
 int	anni_adam_bind_grad(anni_adam *opt, void *d_grad);
 /* gpu_adam_seed_bf16_flat: twins = bf16(p) for the whole flat (after loading weights). */
 int	anni_adam_seed_twins(anni_adam *opt);

@@ -40,12 +40,12 @@ def twin_mask(opt):
 
 
 def run_fp32_case(gpu, oracle, tensors, steps, clip, wd, gmul, grad_scale=1.0, seed=0,
-                  sched=(100, 1000, "cosine")):
+                  sched=(100, 1000, "cosine"), layout=0):
     """Ten steps on the arena vs the oracle twice: against the oracle's own (serial) norm with the
     BASELINE tolerances, and bit for bit when the oracle is handed the device's sum of squares."""
     from anni_amd import lm_adam
     rng = np.random.default_rng(seed)
-    opt = make(gpu, tensors, beta2=0.95, weight_decay=wd, grad_clip=clip)
+    opt = make(gpu, tensors, beta2=0.95, weight_decay=wd, grad_clip=clip, layout=layout)
     n = opt.n
     p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
     opt.upload("param", p0)
@@ -87,6 +87,20 @@ def run_fp32_case(gpu, oracle, tensors, steps, clip, wd, gmul, grad_scale=1.0, s
             assert st.last_grad_scale == OB.o.last_grad_scale
     opt.free()
     return n_clipped
+
+
+def test_spread_layout_gives_the_same_results(gpu, oracle):
+    """Every flat in its own 16 GiB region of device memory (one 80 GiB allocation)."""
+    from anni_amd import lib
+    opt = make(gpu, RAGGED, layout=lib.LAYOUT_SPREAD, grad_slots=2)
+    assert opt.spread and opt.grad_slot(1) - opt.grad_slot(0) >= 4 * opt.n
+    assert opt.o.d_m - opt.o.d_param == 16 << 30 and opt.o.d_v - opt.o.d_m == 16 << 30
+    assert opt.grad_slot(2) is None
+    opt.free()
+    n = sum(t[0] for t in RAGGED)
+    base = 1.0 / (np.sqrt(n) * 1e-3)
+    assert run_fp32_case(gpu, oracle, RAGGED, 4, clip=1.0, wd=0.1, gmul=[0.5 * base, 2.0 * base],
+                         layout=lib.LAYOUT_SPREAD) == 2
 
 
 def test_config1_no_clip_ragged(gpu, oracle):
