@@ -94,6 +94,16 @@ __global__ __launch_bounds__(kThreads) void fp8_quantize_kernel(uint8_t *q, cons
 		q[i] = (uint8_t)fp8_e4m3_encode(x[i] * inv);
 }
 
+/* dst[i] = src[i] over n16 16-byte words: a plain copy of known size (counter calibration). */
+__global__ __launch_bounds__(kThreads) void copy16_kernel(void *dst, const void *src, size_t n16)
+{
+	typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+	const size_t stride = (size_t)gridDim.x * kThreads;
+
+	for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n16; i += stride)
+		((u32x4 *)dst)[i] = ((const u32x4 *)src)[i];
+}
+
 static int util_grid(int64_t items)
 {
 	int64_t g = (items + kThreads - 1) / kThreads;
@@ -126,6 +136,16 @@ int anni_f32_to_bf16(void *d_dst, const float *d_src, int64_t n)
 	if (!d_dst || !d_src || n <= 0 || !device_ready())
 		return -1;
 	return launch_f32_to_bf16(compute_stream(), (uint16_t *)d_dst, d_src, n);
+}
+
+int anni_copy_bytes(void *d_dst, const void *d_src, size_t nbytes)
+{
+	if (!d_dst || !d_src || nbytes == 0 || (nbytes & 15) || ((uintptr_t)d_dst & 15)
+	    || ((uintptr_t)d_src & 15) || !device_ready())
+		return -1;
+	hipLaunchKernelGGL(copy16_kernel, dim3(util_grid((int64_t)(nbytes / 16))), dim3(kThreads), 0,
+	    compute_stream(), d_dst, d_src, nbytes / 16);
+	return hip_ok(hipGetLastError(), "copy_bytes") ? 0 : -1;
 }
 
 int anni_fp8_quantize(void *d_q, float *d_scale, const float *d_src, int64_t n)

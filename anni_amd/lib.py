@@ -98,6 +98,7 @@ _PROTOS = {
     "anni_gpu_set_stream": (None, [C.c_void_p]),
     "anni_fill_normal_f32": (C.c_int, [C.c_void_p, C.c_int64, C.c_uint64, C.c_uint64,
                                        C.c_float, C.c_float]),
+    "anni_copy_bytes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "anni_f32_to_bf16": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64]),
     "anni_fp8_quantize": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]),
 }

@@ -36,6 +36,9 @@ WORKLOADS = {
     "1p4b-fp8": ("1p4b", 2, 0, 1, 28),      # BASELINE config 5
 }
 ELEM = {0: 4, 1: 2, 2: 1}
+# HBM bytes per launch of the update kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled
+# by what the counter reads for a plain copy kernel of known size (summaries under profiles/).
+TRAFFIC_BYTES = {"555m": 18903090561}
 STORAGE = {"185m": "f32 p/g/m/v + bf16 twin", "555m": "f32 p/g/m/v + bf16 twin",
            "555m-bf16": "f32 p, bf16 g/m/v + bf16 twin",
            "1p4b-fp8": "f32 p/m/v, fp8-e4m3 g with per-tensor scale + bf16 twin"}
@@ -89,8 +92,9 @@ def cpu_baselines(size_name, norm_bpp, upd_bpp, budget_s):
     p, g0 = sample(n)
     m = np.zeros(n, np.float32)
     v = np.zeros(n, np.float32)
+    simd = ob.cpu_simd()
     O = ob.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, threads=threads,
-                  norm_threads=threads)
+                  norm_threads=threads, simd=simd)
     g = g0.copy()
     O.step(p, g, m, v, 3e-6, 1.0 / (math.sqrt(n) * 1e-3) * 1.7)      # warm the pages
     times = []
@@ -106,8 +110,11 @@ def cpu_baselines(size_name, norm_bpp, upd_bpp, budget_s):
     mt = float(np.median(times))
     mt_out = {
         "value": round(n * bpp / mt / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        "simd": simd,
         "sample": "first %d of %d params of the workload, %d timed steps (median), fp32 state, "
-                  "clip 1.0 + decay 0.1, OpenMP over %d threads" % (n, n_full, len(times), threads),
+                  "clip 1.0 + decay 0.1, OpenMP over %d threads, %s build (gcc -O3 auto-vectorised, "
+                  "no FMA contraction: bit-identical to the serial loop)"
+                  % (n, n_full, len(times), threads, simd),
         "params_per_s": round(n / mt, 1), "ms_per_step_sample": round(mt * 1e3, 3),
         "ms_per_step_extrapolated": round(mt * 1e3 * n_full / n, 1),
     }
@@ -152,6 +159,22 @@ def cpu_baselines(size_name, norm_bpp, upd_bpp, budget_s):
     return mt_out, serial_out
 
 
+def copy_calibration(L, nbytes):
+    """Ten launches of the plain copy kernel: each reads nbytes and writes nbytes exactly."""
+    from anni_amd.lm_adam import DeviceBuffer
+    nbytes = nbytes // 16 * 16
+    src, dst = DeviceBuffer(nbytes), DeviceBuffer(nbytes)
+    assert L.gpu_memset(src.ptr, 1, nbytes) == 0 and L.gpu_memset(dst.ptr, 0, nbytes) == 0
+    L.gpu_device_sync()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        assert L.anni_copy_bytes(dst.ptr, src.ptr, nbytes) == 0
+    L.gpu_device_sync()
+    ms = (time.perf_counter() - t0) * 1e3 / 10
+    print(json.dumps({"copy_bytes": nbytes, "launches": 10, "ms_per_launch": round(ms, 4),
+                      "GBps_read_plus_write": round(2 * nbytes / ms / 1e6, 1)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -161,6 +184,8 @@ def main():
     ap.add_argument("--layout", default="auto", choices=["auto", "compact", "spread"],
                     help="arena layout (spread: every flat in its own 16 GiB region)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
+                    help="only run the plain copy kernel over BYTES ten times (counter calibration)")
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds for the CPU legs")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -172,6 +197,9 @@ def main():
     from anni_amd import layout, lib
     from anni_amd.lm_adam import LmAdam
     L = lib.require_gpu()
+    if a.copy_calibration:
+        copy_calibration(L, a.copy_calibration)
+        return
 
     size, gt, mt, norm_bpp, upd_bpp = WORKLOADS[a.workload]
     tensors = layout.tensors(size)
@@ -248,7 +276,8 @@ def main():
         "event_ms_per_step": round(ev_ms / a.steps, 4),
         "roofline": {"bound": "hbm", "kernel": "adam_update_kernel", "achieved": round(upd_gbps, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(upd_gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(upd_gbps / HBM_PEAK_GBPS, 4),
+                     "traffic": TRAFFIC_BYTES.get(a.workload),
                      "bytes_per_launch": n * upd_bpp, "avg_ms": round(upd_ms, 4)},
         "sumsq_kernel": {"avg_ms": round(sumsq_ms, 4), "bytes_per_launch": n * norm_bpp,
                          "achieved": round(n * norm_bpp / (sumsq_ms * 1e-3) / 1e9, 1)

@@ -157,6 +157,8 @@ int	anni_adam_time_steps(anni_adam *opt, int count, void *const *grads, int n_gr
 /* x[i] = mean + std * N(0,1), counter-based (seed, stream, i): same values for any launch shape. */
 int	anni_fill_normal_f32(float *d_x, int64_t n, uint64_t seed, uint64_t stream,
 		float mean, float std);
+/* Plain 16-byte-vector copy kernel of nbytes (a multiple of 16, 16-byte aligned): reads and writes exactly nbytes. */
+int	anni_copy_bytes(void *d_dst, const void *d_src, size_t nbytes);
 /* dst = bf16(src) round to nearest even (num/gpu_cuda.cu:1497-1513). */
 int	anni_f32_to_bf16(void *d_dst, const float *d_src, int64_t n);
 /*

@@ -36,19 +36,35 @@ class OracleAdam(C.Structure):
 
 def build(force=False):
     """Compile liboracle.so (and _ref when the reference tree is present)."""
-    if force or not os.path.exists(ORACLE_SO):
+    if force or not all(os.path.exists(os.path.join(HERE, f)) for f in
+                        ("liboracle.so", "liboracle_avx2.so", "liboracle_avx512.so")):
         subprocess.check_call(["make", "-C", HERE, "-s"] + (["-B"] if force else []))
 
 
-_lib = None
+_libs = {}
 
 
-def lib():
-    global _lib
-    if _lib is None:
-        if not os.path.exists(ORACLE_SO):
+def cpu_simd():
+    """Widest of avx512 / avx2 / none that this CPU runs."""
+    try:
+        flags = open("/proc/cpuinfo").read()
+    except OSError:
+        return "none"
+    if " avx512f" in flags and " avx512dq" in flags:
+        return "avx512"
+    if " avx2" in flags:
+        return "avx2"
+    return "none"
+
+
+def lib(simd="none"):
+    """The oracle library; simd = "avx2" / "avx512" selects the auto-vectorised build of the
+    same source (bit-identical results, used for the CPU timing leg)."""
+    so = ORACLE_SO if simd == "none" else os.path.join(HERE, "liboracle_%s.so" % simd)
+    if so not in _libs:
+        if not os.path.exists(so):
             build()
-        L = C.CDLL(ORACLE_SO)
+        L = C.CDLL(so)
         L.oracle_adam_defaults.argtypes = [C.POINTER(OracleAdam), C.c_int64]
         L.oracle_adam_step_scaled.argtypes = [
             C.POINTER(OracleAdam), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
@@ -75,8 +91,8 @@ def lib():
             C.c_void_p, C.c_int64, C.c_int, C.c_double, C.c_double, C.c_double,
             C.c_double, C.c_double, C.c_double, C.c_double]
         L.oracle_max_threads.restype = C.c_int
-        _lib = L
-    return _lib
+        _libs[so] = L
+    return _libs[so]
 
 
 def _ptr(a):
@@ -96,8 +112,9 @@ class Oracle:
 
     def __init__(self, n, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0,
                  grad_clip=0.0, skip_nonfinite=False, grad_type=F32, moment_type=F32,
-                 tensors=None, threads=1, norm_threads=1):
+                 tensors=None, threads=1, norm_threads=1, simd="none"):
         self.o = OracleAdam()
+        self.L = lib(simd)
         lib().oracle_adam_defaults(C.byref(self.o), n)
         self.o.beta1, self.o.beta2, self.o.eps = beta1, beta2, eps
         self.o.weight_decay, self.o.grad_clip = weight_decay, grad_clip
@@ -116,7 +133,7 @@ class Oracle:
         ov = None
         if sumsq_override is not None:
             ov = C.byref(C.c_double(float(sumsq_override)))
-        return lib().oracle_adam_step_scaled(
+        return self.L.oracle_adam_step_scaled(
             C.byref(self.o), _ptr(p), _ptr(g), _ptr(m), _ptr(v), _ptr(twin),
             self.segs, self.nsegs, lr, grad_scale, ov, self.threads)
 

@@ -20,11 +20,22 @@ def same_bits(a, b):
 
 
 def rel_err(a, b):
-    """max |a-b| / max(|b|, tiny) over finite entries, in double."""
+    """max |a-b| / max(|b|, rms(b)), in double.
+
+    Used only where the two sides were computed under clip norms that differ in their last
+    bits (different summation order).  m = b1*m + (1-b1)*g cancels for some elements, and there
+    ANY perturbation of the gradient scale -- the 1e-5 the norm itself is allowed included --
+    is amplified without bound relative to the tiny result, and one float ulp of m carried into
+    the next step does the same.  Errors are therefore measured against max(|b|, rms(b)): relative
+    for ordinary elements, against the array's own scale for cancelling ones.  Where both sides
+    use the same norm the tests ask for identical bits instead.
+    """
+    if not a.size:
+        return 0.0
     a = a.astype(np.float64)
     b = b.astype(np.float64)
-    den = np.maximum(np.abs(b), 1e-30)
-    return float(np.max(np.abs(a - b) / den)) if a.size else 0.0
+    floor = float(np.sqrt(np.mean(b * b))) + 1e-300
+    return float(np.max(np.abs(a - b) / np.maximum(np.abs(b), floor)))
 
 
 def bf16_ulp_diff(a_u16, b_u16):

@@ -76,6 +76,30 @@ def test_oracle_matches_golden(oracle, name, threads):
         assert not g.any()
 
 
+@pytest.mark.parametrize("simd", ["avx2", "avx512"])
+def test_vectorised_build_is_bit_identical(oracle, simd):
+    """The -O3 auto-vectorised build of the same source (CPU timing leg) vs the reference-flags build."""
+    if simd == "avx512" and oracle.cpu_simd() != "avx512":
+        pytest.skip("CPU without AVX-512")
+    if simd == "avx2" and oracle.cpu_simd() == "none":
+        pytest.skip("CPU without AVX2")
+    rng = np.random.default_rng(17)
+    n = 300007
+    p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    A = dict(p=p0.copy(), m=np.zeros(n, np.float32), v=np.zeros(n, np.float32))
+    B = dict(p=p0.copy(), m=np.zeros(n, np.float32), v=np.zeros(n, np.float32))
+    OA = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0)
+    OB = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, threads=4, simd=simd)
+    for s in range(5):
+        g = (rng.standard_normal(n) * 1e-3 * (1 + 3 * (s % 2))).astype(np.float32)
+        ga, gb = g.copy(), g.copy()
+        OA.step(A["p"], ga, A["m"], A["v"], 3e-4)
+        OB.step(B["p"], gb, B["m"], B["v"], 3e-4)
+        assert OA.o.last_sumsq == OB.o.last_sumsq        # serial norm in both
+        for k in "pmv":
+            assert same_bits(A[k], B[k]), (simd, s, k)
+
+
 def test_golden_lr_table(oracle):
     T = np.load(__import__("os").path.join(__import__("helpers").GOLDEN, "lr_table.npz"))
     for row, case in zip(T["lr"], T["cases"]):
