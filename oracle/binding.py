@@ -237,3 +237,69 @@ class RefAdam:
 
 def ref_lr(base_lr, step, warmup=0, decay_steps=0, kind="none", sched_from=0):
     return ref().ref_step_lr(base_lr, step, warmup, decay_steps, kind.encode(), sched_from)
+
+
+# ---- the reference's compiled optimizer linked against THIS repository's HIP backend ----
+
+REF_HIP_SO = os.path.join(HERE, "_ref", "libanni_ref_hip.so")
+_ref_hip = None
+
+
+def ref_hip_available():
+    return os.path.exists(REF_HIP_SO)
+
+
+def ref_hip():
+    global _ref_hip
+    if _ref_hip is None:
+        R = C.CDLL(REF_HIP_SO)
+        R.ref_adam_create_device.argtypes = [C.c_void_p, C.c_void_p, C.c_long, C.c_double,
+                                             C.c_double, C.c_double, C.c_double, C.c_double]
+        R.ref_adam_create_device.restype = C.c_void_p
+        R.ref_adam_step.argtypes = [C.c_void_p, C.c_double, C.c_double]
+        R.ref_adam_step.restype = C.c_int
+        R.ref_adam_sync_host.argtypes = [C.c_void_p]
+        R.ref_adam_last_norm.argtypes = [C.c_void_p]
+        R.ref_adam_last_norm.restype = C.c_double
+        R.ref_adam_on_device.argtypes = [C.c_void_p]
+        R.ref_adam_on_device.restype = C.c_int
+        R.ref_adam_release_device.argtypes = [C.c_void_p]
+        R.ref_adam_export.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        R.ref_adam_free.argtypes = [C.c_void_p]
+        _ref_hip = R
+    return _ref_hip
+
+
+class RefAdamOnBackend:
+    """The unchanged lm_adam_step_scaled taking its device path on libanni_gpu_hip.so."""
+
+    def __init__(self, p, g, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0, grad_clip=0.0):
+        self.p, self.g = p, g
+        self.h = ref_hip().ref_adam_create_device(_ptr(p), _ptr(g), p.size, beta1, beta2, eps,
+                                                  weight_decay, grad_clip)
+        if not self.h:
+            raise MemoryError("ref_adam_create_device")
+
+    def step(self, lr, grad_scale=1.0):
+        return ref_hip().ref_adam_step(self.h, lr, grad_scale)
+
+    @property
+    def last_grad_norm(self):
+        return ref_hip().ref_adam_last_norm(self.h)
+
+    @property
+    def on_device(self):
+        return bool(ref_hip().ref_adam_on_device(self.h))
+
+    def moments(self):
+        ref_hip().ref_adam_sync_host(self.h)
+        m = np.empty(self.p.size, dtype=np.float32)
+        v = np.empty(self.p.size, dtype=np.float32)
+        ref_hip().ref_adam_export(self.h, _ptr(m), _ptr(v))
+        return m, v
+
+    def close(self):
+        if self.h:
+            ref_hip().ref_adam_release_device(self.h)
+            ref_hip().ref_adam_free(self.h)
+            self.h = None

@@ -10,6 +10,7 @@
 */
 #include <stdlib.h>
 #include <string.h>
+#include "gpu.h"
 #include "lm_adam.h"
 #include "lm_train.h"
 
@@ -17,6 +18,9 @@ typedef struct ref_adam {
 	lm_adam	opt;
 	float	*p;
 	float	*g;
+	vec	wv;	/* one bias-style segment over the whole flat (device path only) */
+	vec	dwv;
+	lm_adam_seg	seg;
 } ref_adam;
 
 ref_adam *ref_adam_create(float *p, float *g, const float *m, const float *v, long n,
@@ -48,6 +52,66 @@ ref_adam *ref_adam_create(float *p, float *g, const float *m, const float *v, lo
 	r->p = p;
 	r->g = g;
 	return r;
+}
+
+/*
+** Same, but registered as one host-resident vector segment (the kind lm_adam.c keeps for
+** biases and LayerNorm vectors, lm_adam.c:43-57): when the library is linked against a real
+** backend, lm_adam_step_scaled then takes its DEVICE path (lm_adam.c:452-515) -- gpu_malloc,
+** H2D gather, gpu_grad_sumsq, clip, gpu_adam_step_dev_bf16, async D2H scatter -- unchanged.
+*/
+ref_adam *ref_adam_create_device(float *p, float *g, long n, double beta1, double beta2,
+	double eps, double wd, double clip)
+{
+	ref_adam *r = ref_adam_create(p, g, NULL, NULL, n, 0, beta1, beta2, eps, wd, clip);
+
+	if (!r)
+		return NULL;
+	r->wv.data = p;
+	r->wv.n = (int)n;
+	r->dwv.data = g;
+	r->dwv.n = (int)n;
+	r->seg.wv = &r->wv;
+	r->seg.dwv = &r->dwv;
+	r->seg.off = 0;
+	r->seg.n = (int)n;
+	r->opt.segs = &r->seg;
+	r->opt.n_segs = 1;
+	return r;
+}
+
+/* Pulls the device-resident moments into the slots (lm_adam.c:336-358). */
+void ref_adam_sync_host(ref_adam *r)
+{
+	lm_adam_sync_host(&r->opt);
+}
+
+double ref_adam_last_norm(const ref_adam *r)
+{
+	return r->opt.last_grad_norm;
+}
+
+int ref_adam_on_device(const ref_adam *r)
+{
+	return r->opt.d_param != NULL;
+}
+
+/* Frees the device flats the reference allocated (what lm_adam_free does, lm_adam.c:185-194). */
+void ref_adam_release_device(ref_adam *r)
+{
+	if (r->opt.d_param) {
+		gpu_adam_set_bf16_flat(NULL, NULL, 0);
+		gpu_free(r->opt.d_param);
+		gpu_free(r->opt.d_param_bf16);
+		gpu_free(r->opt.d_grad);
+		gpu_free(r->opt.d_m);
+		gpu_free(r->opt.d_v);
+		free(r->opt.h_m);
+		free(r->opt.h_v);
+		r->opt.d_param = r->opt.d_grad = r->opt.d_m = r->opt.d_v = NULL;
+		r->opt.d_param_bf16 = NULL;
+		r->opt.h_m = r->opt.h_v = NULL;
+	}
 }
 
 /* Returns opt->t after the call. */

@@ -309,3 +309,45 @@ def test_seed_bf16_flat(gpu, oracle):
         assert (o.download(np.uint16, n) == oracle.bf16_rne(x)).all()
         gpu.gpu_adam_set_bf16_flat(None, None, 0)
     assert gpu.gpu_adam_seed_bf16_flat(None, None, 5) == -1
+
+
+def test_the_unchanged_reference_caller_on_this_backend(gpu, oracle):
+    """lang/lm_adam.c itself, compiled from the reference tree and linked against
+    libanni_gpu_hip.so instead of its CPU stub (oracle/_ref/libanni_ref_hip.so): its device path
+    (lm_adam.c:452-515) runs on this backend and must give what its own host path gives."""
+    if not oracle.ref_hip_available():
+        pytest.skip("oracle/_ref/libanni_ref_hip.so not built (reference tree absent at build time)")
+    rng = np.random.default_rng(2024)
+    n = 200003
+    p = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    g = np.zeros(n, np.float32)
+    P, M, V = p.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    gpu.gpu_set_compute_prec(1)
+    e0 = gpu.gpu_param_epoch()
+    R = oracle.RefAdamOnBackend(p, g, beta2=0.95, weight_decay=0.1, grad_clip=1.0)
+    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1)            # clip applied by hand below
+    Ocpu = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0)
+    Pc, Mc, Vc = p.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    unit = 1.0 / (math.sqrt(n) * 1e-3)
+    for t in range(1, 11):
+        gg = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+        g[:] = gg
+        lr = oracle.lr(3e-4, t - 1, 100, 1000, "cosine")
+        gs = unit * (1.7 if t % 2 else 0.6)
+        assert R.step(lr, gs) == t and R.on_device
+        # the caller's own device-branch arithmetic: norm = sqrt(ss)*|gs|, scale *= clip/norm
+        norm = R.last_grad_norm
+        eff = gs * (1.0 / norm) if norm > 1.0 else gs
+        O.step(P, gg.copy(), M, V, lr, eff)
+        m, v = R.moments()
+        assert same_bits(p, P) and same_bits(m, M) and same_bits(v, V), t
+        assert not g.any()                                          # vec_zero after the scatter
+        # ... and against the caller's HOST path (clip/(norm+1e-12), serial norm): tolerances
+        Ocpu.step(Pc, gg.copy(), Mc, Vc, lr, gs)
+        assert abs(norm - Ocpu.o.last_grad_norm) <= TOL_NORM * norm
+        assert rel_err(p, Pc) <= TOL_STATE and rel_err(m, Mc) <= TOL_STATE
+        assert rel_err(v, Vc) <= TOL_STATE
+    assert gpu.gpu_param_epoch() >= e0 + 10
+    R.close()
+    gpu.gpu_set_compute_prec(0)
+    gpu.gpu_adam_set_weight_decay(0.0)
