@@ -84,34 +84,68 @@ struct Placement {
 };
 
 /*
-** Layout.  On MI355X a kernel that streams several arrays at once runs about 20 %
-** faster when the arrays lie in different 16 GiB regions of device memory than when two
-** of them share one (measured: 6.2 against 5.1 TB/s for this update; a kernel with a
-** single stream does not care).  SPREAD therefore puts p, m, v and the twins one region
-** apart and the gradient slots behind them, all inside ONE allocation whose size is a
-** whole number of regions, so same-index elements of any two flats are a whole number
-** of regions apart.  The holes are reserved with it.  COMPACT packs the flats at 2 MiB
-** boundaries.
+** Layout.  On MI355X a kernel that streams several arrays at once runs about 20 % faster
+** when the arrays lie in different 16 GiB regions of device memory than when two of them
+** share one (measured: 6.2 against 5.1 TB/s for this update; a kernel with a single
+** stream does not care), and another 4 % faster when no more than three of them lie in
+** the same group of four regions.  SPREAD therefore uses ONE allocation of a whole number
+** of regions: p, m, v in regions 0, 1, 2, the twins in region 4, the gradient slots from
+** region 5 on (region 3 holds only the small tables), so same-index elements of any two
+** flats are a whole number of regions apart.  The holes are reserved with it.  COMPACT
+** packs the flats at 2 MiB boundaries.
 */
+/*
+** Size of a spread arena.  The driver hands out device memory in naturally aligned
+** power-of-two blocks.  Up to six regions the arena is a 4-region block plus a 2-region
+** block (the layout keeps three flats in each); beyond that it is rounded up to one
+** power-of-two block, because a third, stray block was measured to make the gradient
+** slots that land in it 10 % slower than the others.
+*/
+static size_t spread_total(size_t need)
+{
+	size_t p2 = region_bytes();
+
+	need = round_up(need, region_bytes());
+	if (need <= 6 * region_bytes())
+		return need;
+	while (p2 < need)
+		p2 <<= 1;
+	return p2;
+}
+
 static bool place(const Sizes &z, bool spread, Placement *pl)
 {
 	const size_t big = (size_t)2 << 20;
 	const size_t stride = spread ? round_up(z.p_bytes, region_bytes()) : 0;
+	const size_t tables = round_up((size_t)z.n_tensors * sizeof(float), 256)
+	    + round_up((size_t)z.n_tensors * sizeof(Seg), 256)
+	    + round_up((size_t)z.n_tiles * sizeof(int32_t), 256)
+	    + round_up((size_t)kMaxPartials * sizeof(double), 256) + 256;
 
 	memset(pl, 0, sizeof(*pl));
-	pl->off_p = 0;
-	pl->off_m = spread ? stride : round_up(pl->off_p + z.p_bytes, big);
-	pl->off_v = spread ? 2 * stride : round_up(pl->off_m + z.mv_bytes, big);
-	pl->off_twin = spread ? 3 * stride : round_up(pl->off_v + z.mv_bytes, big);
-	pl->off_g = spread ? 4 * stride : round_up(pl->off_twin + z.tw_bytes, big);
-	pl->off_gscale = round_up(pl->off_g + (size_t)z.n_slots * z.g_bytes, big);
+	if (spread) {
+		pl->off_p = 0;
+		pl->off_m = stride;
+		pl->off_v = 2 * stride;
+		pl->off_gscale = 3 * stride;		/* tables */
+		pl->off_twin = 4 * stride;
+		pl->off_g = (z.tw_bytes ? 5 : 4) * stride;
+		pl->total = spread_total(pl->off_g + (size_t)z.n_slots * z.g_bytes + big);
+		if (tables > stride)
+			return false;
+	} else {
+		pl->off_p = 0;
+		pl->off_m = round_up(pl->off_p + z.p_bytes, big);
+		pl->off_v = round_up(pl->off_m + z.mv_bytes, big);
+		pl->off_twin = round_up(pl->off_v + z.mv_bytes, big);
+		pl->off_g = round_up(pl->off_twin + z.tw_bytes, big);
+		pl->off_gscale = round_up(pl->off_g + (size_t)z.n_slots * z.g_bytes, big);
+		pl->total = pl->off_gscale + tables;
+	}
 	pl->off_segs = pl->off_gscale + round_up((size_t)z.n_tensors * sizeof(float), 256);
 	pl->off_tiles = pl->off_segs + round_up((size_t)z.n_tensors * sizeof(Seg), 256);
 	pl->off_part = pl->off_tiles + round_up((size_t)z.n_tiles * sizeof(int32_t), 256);
 	pl->off_state = pl->off_part + round_up((size_t)kMaxPartials * sizeof(double), 256);
-	pl->total = pl->off_state + 256;
-	if (spread)
-		pl->total = round_up(pl->total, region_bytes());
 	pl->spread = spread ? 1 : 0;
 	if (hipMalloc(&pl->arena, pl->total) != hipSuccess) {
 		(void)hipGetLastError();
@@ -197,6 +231,8 @@ static double probe(const anni_adam *opt)
 	c.eps = 1e-8;
 	c.bc1 = c.omb1;
 	c.bc2 = c.omb2;
+	c.rbc1 = 1.0 / c.bc1;
+	c.rbc2 = 1.0 / c.bc2;
 	c.lr = 1e-3;
 	memset(&norm, 0, sizeof(norm));
 	describe(opt, &f);
@@ -227,15 +263,15 @@ anni_adam *anni_adam_create(const anni_tensor *tensors, int n_tensors,
 	const anni_adam_config *cfg)
 {
 	const size_t big = (size_t)2 << 20;	/* each flat starts on a 2 MiB boundary */
-	/* A spread placement is tried again (up to kTries) while the probe stays below kGoodGBps. */
+	/* A spread arena is requested again (up to kTries) while the probe stays below these. */
 	const int kTries = 3;
 	const double kGoodGBps = 5600.0;
+	const double kGoodGBpsNarrow = 5300.0;
 	anni_adam *opt;
 	anni_adam_priv *pv;
 	Sizes z;
 	std::vector<Seg> segs;
 	std::vector<int32_t> tile_seg;
-	std::vector<Placement> tried;
 	Placement pl;
 	int64_t n = 0;
 	bool want_spread;
@@ -321,8 +357,8 @@ anni_adam *anni_adam_create(const anni_tensor *tensors, int n_tensors,
 	want_spread = cfg->layout == ANNI_LAYOUT_SPREAD;
 	if (cfg->layout == ANNI_LAYOUT_AUTO && z.p_bytes >= ((size_t)256 << 20)) {
 		size_t free_b = 0, total_b = 0;
-		const size_t need = round_up(4 * round_up(z.p_bytes, region_bytes())
-		    + (size_t)z.n_slots * z.g_bytes + ((size_t)64 << 20), region_bytes());
+		const size_t need = spread_total(5 * round_up(z.p_bytes, region_bytes())
+		    + (size_t)z.n_slots * z.g_bytes + ((size_t)64 << 20));
 
 		if (hipMemGetInfo(&free_b, &total_b) == hipSuccess && need <= free_b / 2)
 			want_spread = true;
@@ -330,36 +366,33 @@ anni_adam *anni_adam_create(const anni_tensor *tensors, int n_tensors,
 	}
 	if (want_spread) {
 		/*
-		** Where a placement lands physically is the driver's choice and it shows in the
-		** throughput, so a slow one is kept aside (which makes the next one land
-		** elsewhere) and the fastest of a few is used.  Only with gradient slots to run on.
+		** What the driver backs an allocation with is its choice and shows in the
+		** throughput: right after other large allocations were freed a new one can be
+		** slow as a whole (every placement inside it), and the same request a moment
+		** later is fine.  So the update is timed on the fresh arena and a slow arena is
+		** FREED and requested again, a few times.  Needs gradient slots to run on.
 		*/
 		const bool audition = z.n_slots > 0 && z.p_bytes >= ((size_t)256 << 20);
+		const double good = cfg->moment_type == ANNI_F32 ? kGoodGBps : kGoodGBpsNarrow;
 
-		for (int k = 0; k < kTries; k++) {
+		for (int k = 0; k < kTries && !ok; k++) {
 			if (!place(z, true, &pl))
 				break;
 			adopt(opt, z, pl);
 			if (!init_contents(opt, z, pl, segs, tile_seg)) {
 				(void)hipFree(pl.arena);
+				pv->arena = nullptr;
 				break;
 			}
 			pl.gbps = audition ? probe(opt) : 0.0;
-			tried.push_back(pl);
-			if (!audition || pl.gbps >= kGoodGBps)
-				break;
-		}
-		if (!tried.empty()) {
-			size_t best = 0;
-
-			for (size_t k = 1; k < tried.size(); k++)
-				if (tried[k].gbps > tried[best].gbps)
-					best = k;
-			for (size_t k = 0; k < tried.size(); k++)
-				if (k != best)
-					(void)hip_ok(hipFree(tried[k].arena), "arena hipFree");
-			adopt(opt, z, tried[best]);
-			ok = true;
+			pv->probe_gbps = pl.gbps;
+			if (!audition || pl.gbps >= good || k == kTries - 1) {
+				ok = true;
+			} else {
+				(void)hipStreamSynchronize(compute_stream());
+				(void)hip_ok(hipFree(pl.arena), "arena hipFree");
+				pv->arena = nullptr;
+			}
 		}
 	}
 	if (!ok && cfg->layout != ANNI_LAYOUT_SPREAD) {
@@ -488,6 +521,8 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 	c.bc2 = 1.0 - pow(opt->beta2, (double)opt->t);
 	if (c.bc1 <= 0.0 || c.bc2 <= 0.0)
 		return -1;			/* gpu_cuda.cu:8681-8682 */
+	c.rbc1 = 1.0 / c.bc1;
+	c.rbc2 = 1.0 / c.bc2;
 	c.beta1 = opt->beta1;
 	c.omb1 = 1.0 - opt->beta1;
 	c.beta2 = opt->beta2;

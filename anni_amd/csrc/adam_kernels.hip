@@ -56,10 +56,13 @@ __device__ __forceinline__ f32x4 load_quad(const void *base, int64_t i, float sc
 	} else {
 		const uint32_t w = ld<NT>((const uint32_t *)((const uint8_t *)base + i));
 
-		r.x = fp8_e4m3_decode(w & 0xffu) * scale;
-		r.y = fp8_e4m3_decode((w >> 8) & 0xffu) * scale;
-		r.z = fp8_e4m3_decode((w >> 16) & 0xffu) * scale;
-		r.w = fp8_e4m3_decode(w >> 24) * scale;
+		const f32x2_t lo = fp8_e4m3_decode2(w, false);
+		const f32x2_t hi = fp8_e4m3_decode2(w, true);
+
+		r.x = lo.x * scale;
+		r.y = lo.y * scale;
+		r.z = hi.x * scale;
+		r.w = hi.y * scale;
 	}
 	return r;
 }
@@ -255,6 +258,89 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(SumsqArgs a)
 		a.partials[blockIdx.x] = total;
 }
 
+/*
+** FP8 gradients: sum = SUM over tensors of (scale_t * gs)^2 * SUM_i decode(q_i)^2.  The square
+** of an E4M3 value is exact in float and the inner sums are exact in double, so only the
+** per-tile products round.  One 16-byte load (16 codes) per lane per tile, four tiles in flight.
+*/
+template <bool NT>
+__global__ __launch_bounds__(kThreads) void sumsq_fp8_kernel(SumsqArgs a)
+{
+	typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+	__shared__ double lds[4];
+	constexpr int kAhead = 4;
+	const int tid = threadIdx.x;
+	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
+	double acc = 0.0;
+
+	for (int64_t t0 = blockIdx.x; t0 < n_tiles; t0 += (int64_t)gridDim.x * kAhead) {
+		u32x4 W[kAhead];
+		double s2[kAhead];
+		bool fast[kAhead];
+
+#pragma unroll
+		for (int j = 0; j < kAhead; j++) {
+			const int64_t tile = t0 + (int64_t)j * gridDim.x;
+
+			fast[j] = false;
+			s2[j] = 0.0;
+			W[j] = u32x4{0u, 0u, 0u, 0u};
+			if (tile < n_tiles) {
+				const int64_t base = tile * kTile;
+				const int64_t end = base + kTile < a.n ? base + kTile : a.n;
+				const int s = a.tile_seg ? a.tile_seg[tile] : 0;
+				const int64_t seg_end = a.segs ? a.segs[s].end : a.n;
+
+				if (a.vec_ok && end - base == kTile && seg_end >= end) {
+					const double sc = (double)a.gscale[s] * a.grad_scale;
+
+					fast[j] = true;
+					s2[j] = sc * sc;
+					W[j] = ld<NT>((const u32x4 *)((const uint8_t *)a.g + base) + tid);
+				}
+			}
+		}
+#pragma unroll
+		for (int j = 0; j < kAhead; j++) {
+			const int64_t tile = t0 + (int64_t)j * gridDim.x;
+
+			if (fast[j]) {
+				double t = 0.0;
+
+#pragma unroll
+				for (int k = 0; k < 4; k++) {
+					const f32x2_t lo = fp8_e4m3_decode2(W[j][k], false);
+					const f32x2_t hi = fp8_e4m3_decode2(W[j][k], true);
+
+					t += (double)(lo.x * lo.x);
+					t += (double)(lo.y * lo.y);
+					t += (double)(hi.x * hi.x);
+					t += (double)(hi.y * hi.y);
+				}
+				acc += s2[j] * t;
+			} else if (tile < n_tiles) {
+				const int64_t base = tile * kTile;
+				const int64_t end = base + kTile < a.n ? base + kTile : a.n;
+				int s = a.tile_seg ? a.tile_seg[tile] : 0;
+
+				for (int64_t i = base + tid; i < end; i += kThreads) {
+					if (a.segs)
+						while (i >= a.segs[s].end)
+							s++;
+					const double sc = (double)a.gscale[s] * a.grad_scale;
+					const float d = fp8_e4m3_decode(((const uint8_t *)a.g)[i]);
+
+					acc += (sc * sc) * (double)(d * d);
+				}
+			}
+		}
+	}
+	const double total = block_sum(acc, lds);
+
+	if (tid == 0)
+		a.partials[blockIdx.x] = total;
+}
+
 struct FinalizeArgs {
 	const double	*partials;
 	int		n_partials;
@@ -298,7 +384,11 @@ struct UpdateArgs {
 	StepState	*state;
 };
 
-/* U = quads a lane keeps in flight at once (kQuadsPerTile % U == 0). */
+/*
+** U = quads a lane keeps in flight at once (kQuadsPerTile % U == 0).  With narrow storage
+** types the kernel moves fewer bytes per element for the same arithmetic, so those modes
+** take the cheaper constant division (adam_math.h) and the deeper unroll.
+*/
 template <int GT, int MT, int U, bool NT>
 __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 {
@@ -362,8 +452,8 @@ __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 				for (int u = 0; u < U; u++) {
 #pragma unroll
 					for (int k = 0; k < kQuad; k++) {
-						const Elem e = adam_elem(P[u][k], G[u][k], M[u][k], V[u][k],
-						    gs, a.c, decay);
+						const Elem e = adam_elem<(GT != kF32 || MT != kF32)>(P[u][k],
+						    G[u][k], M[u][k], V[u][k], gs, a.c, decay);
 
 						P[u][k] = e.p;
 						M[u][k] = e.m;
@@ -392,7 +482,7 @@ __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 				}
 				if (GT == kFP8)
 					sc = a.gscale[s];
-				const Elem e = adam_elem(a.p[i], load_one<GT>(a.g, i, sc),
+				const Elem e = adam_elem<(GT != kF32 || MT != kF32)>(a.p[i], load_one<GT>(a.g, i, sc),
 				    load_one<MT>(a.m, i, 1.0f), load_one<MT>(a.v, i, 1.0f), gs, a.c,
 				    a.c.decay_on && (flags & kSegDecay) != 0);
 
@@ -564,8 +654,13 @@ int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *parti
 		SUMSQ_LAUNCH(kF32);
 	else if (f.grad_type == kBF16)
 		SUMSQ_LAUNCH(kBF16);
-	else
-		SUMSQ_LAUNCH(kFP8);
+	else {
+		a.vec_ok = aligned(f.g, 16) ? 1 : 0;
+		if (nt_on())
+			hipLaunchKernelGGL((sumsq_fp8_kernel<true>), dim3(grid), dim3(kThreads), 0, st, a);
+		else
+			hipLaunchKernelGGL((sumsq_fp8_kernel<false>), dim3(grid), dim3(kThreads), 0, st, a);
+	}
 #undef SUMSQ_LAUNCH
 	*n_partials = grid;
 	return hipGetLastError() == hipSuccess ? 0 : -1;
@@ -589,18 +684,23 @@ int launch_finalize(hipStream_t st, const double *partials, int n_partials, doub
 }
 
 #ifndef ANNI_UPDATE_UNROLL
-#define ANNI_UPDATE_UNROLL 2
+#define ANNI_UPDATE_UNROLL 2		/* all-f32 mode */
+#endif
+#ifndef ANNI_UPDATE_UNROLL_NARROW
+#define ANNI_UPDATE_UNROLL_NARROW 4	/* bf16 moments / bf16 or fp8 gradients */
 #endif
 
 template <int GT, int MT>
 static void update_launch(hipStream_t st, int grid, const UpdateArgs &a)
 {
+	constexpr int U = (GT == kF32 && MT == kF32) ? ANNI_UPDATE_UNROLL : ANNI_UPDATE_UNROLL_NARROW;
+
 	if (nt_on())
-		hipLaunchKernelGGL((adam_update_kernel<GT, MT, ANNI_UPDATE_UNROLL, true>),
-		    dim3(grid), dim3(kThreads), 0, st, a);
+		hipLaunchKernelGGL((adam_update_kernel<GT, MT, U, true>), dim3(grid), dim3(kThreads),
+		    0, st, a);
 	else
-		hipLaunchKernelGGL((adam_update_kernel<GT, MT, ANNI_UPDATE_UNROLL, false>),
-		    dim3(grid), dim3(kThreads), 0, st, a);
+		hipLaunchKernelGGL((adam_update_kernel<GT, MT, U, false>), dim3(grid), dim3(kThreads),
+		    0, st, a);
 }
 
 int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double grad_scale,

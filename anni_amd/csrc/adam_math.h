@@ -28,6 +28,8 @@ struct StepConsts {
 	double	lr;
 	double	lr_wd;	/* lr * weight_decay (lm_adam.c:595 multiplies these first) */
 	int	decay_on;	/* weight_decay > 0 (lm_adam.c:594); per-tensor flags select where */
+	double	rbc1;	/* 1.0 / bc1 and 1.0 / bc2, correctly rounded (host division) */
+	double	rbc2;
 };
 
 /* New p, m, v of one element. */
@@ -38,9 +40,24 @@ struct Elem {
 };
 
 /*
+** a / b for a step constant b whose correctly rounded reciprocal rb the host supplies:
+** q = a*rb, then one exact residual a - b*q folded back.  The result is a/b rounded to
+** nearest unless a/b lies within ~2^-52 ulp of a rounding boundary (then it may be the
+** other neighbour): about one quotient in 2^52.  Used only where the update is bound by
+** arithmetic (narrow storage types); the all-f32 mode keeps the IEEE division.
+*/
+__device__ __forceinline__ double div_by_const(double a, double b, double rb)
+{
+	const double q = a * rb;
+
+	return __builtin_fma(__builtin_fma(-b, q, a), rb, q);
+}
+
+/*
 ** g is the gradient element as a float; gs the effective gradient scale.
 ** Rounding points: m, v (float), p after the step, p after the decay.
 */
+template <bool FASTDIV>
 __device__ __forceinline__ Elem adam_elem(float p, float g, float m, float v, double gs,
 	const StepConsts &c, bool decay)
 {
@@ -49,8 +66,8 @@ __device__ __forceinline__ Elem adam_elem(float p, float g, float m, float v, do
 
 	r.m = (float)(c.beta1 * (double)m + c.omb1 * x);
 	r.v = (float)(c.beta2 * (double)v + (c.omb2 * x) * x);
-	const double mhat = (double)r.m / c.bc1;
-	const double vhat = (double)r.v / c.bc2;
+	const double mhat = FASTDIV ? div_by_const((double)r.m, c.bc1, c.rbc1) : (double)r.m / c.bc1;
+	const double vhat = FASTDIV ? div_by_const((double)r.v, c.bc2, c.rbc2) : (double)r.v / c.bc2;
 	r.p = (float)((double)p - (c.lr * mhat) / (sqrt(vhat) + c.eps));
 	if (decay)
 		r.p = (float)((double)r.p - c.lr_wd * (double)r.p);
@@ -88,6 +105,17 @@ __device__ __forceinline__ float fp8_e4m3_decode(uint32_t q)
 	else
 		bits = ((e + 120u) << 23) | (f << 20);
 	return __uint_as_float(s | bits);
+}
+
+/*
+** Two / four OCP E4M3 bytes of a word -> floats with the gfx950 conversion instruction
+** (exact, same values as fp8_e4m3_decode; checked against the table for all 256 codes).
+*/
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ f32x2_t fp8_e4m3_decode2(uint32_t w, bool high)
+{
+	return high ? __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true)
+	    : __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
 }
 
 /* float -> OCP E4M3 byte: round to nearest even, saturate to +-448, NaN -> S.1111.111. */

@@ -473,6 +473,8 @@ int gpu_adam_step_dev_bf16(ann_real *d_param, void *d_param_bf16, ann_real *d_gr
 	c.bc2 = 1.0 - pow(beta2, (double)t);
 	if (c.bc1 <= 0.0 || c.bc2 <= 0.0)
 		return -1;
+	c.rbc1 = 1.0 / c.bc1;
+	c.rbc2 = 1.0 / c.bc2;
 	c.beta1 = beta1;
 	c.omb1 = 1.0 - beta1;
 	c.beta2 = beta2;

@@ -34,6 +34,7 @@ WORKLOADS = {
     "555m": ("555m", 0, 0, 4, 34),          # BASELINE config 3 (headline)
     "555m-bf16": ("555m", 1, 1, 2, 22),     # BASELINE config 4
     "1p4b-fp8": ("1p4b", 2, 0, 1, 28),      # BASELINE config 5
+    "1p4b": ("1p4b", 0, 0, 4, 34),          # the 1.4B set in the all-f32 mode (comparison only)
 }
 ELEM = {0: 4, 1: 2, 2: 1}
 # HBM bytes per launch of the update kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled
@@ -41,7 +42,8 @@ ELEM = {0: 4, 1: 2, 2: 1}
 TRAFFIC_BYTES = {"555m": 18903090561}
 STORAGE = {"185m": "f32 p/g/m/v + bf16 twin", "555m": "f32 p/g/m/v + bf16 twin",
            "555m-bf16": "f32 p, bf16 g/m/v + bf16 twin",
-           "1p4b-fp8": "f32 p/m/v, fp8-e4m3 g with per-tensor scale + bf16 twin"}
+           "1p4b-fp8": "f32 p/m/v, fp8-e4m3 g with per-tensor scale + bf16 twin",
+           "1p4b": "f32 p/g/m/v + bf16 twin"}
 
 
 def fill_grad_slots(L, opt, tensors, count, grad_type, seed):
@@ -178,7 +180,8 @@ def copy_calibration(L, nbytes):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps (default 10 for the headline workload, 8 otherwise)")
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="555m", choices=sorted(WORKLOADS))
     ap.add_argument("--layout", default="auto", choices=["auto", "compact", "spread"],
@@ -188,6 +191,8 @@ def main():
                     help="only run the plain copy kernel over BYTES ten times (counter calibration)")
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds for the CPU legs")
     a = ap.parse_args()
+    if a.steps is None:
+        a.steps = 10 if a.workload == "555m" else 8
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the step has no multi-GPU path); "
                  "use --gpus 1")

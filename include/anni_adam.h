@@ -42,9 +42,10 @@ extern "C" {
 ** (one allocation, holes included), which is what lets a kernel that streams all of
 ** them at once reach full HBM speed on MI355X; COMPACT packs them.  AUTO spreads when
 ** the parameter flat is at least 256 MiB and the spread arena takes less than half of
-** the free device memory.  Where a spread arena lands physically is the driver's choice
-** and shows in the throughput: creation times the update on a few placements and keeps
-** the fastest (only when the arena owns gradient slots to run on).
+** the free device memory.  What the driver backs the allocation with shows in the
+** throughput: creation times the update on the new arena and asks again (up to three
+** times, freeing in between) while it is slow; this needs gradient slots to run on.
+** Reserving and releasing ~100 GiB takes the driver a few seconds.
 */
 #define ANNI_LAYOUT_AUTO	0
 #define ANNI_LAYOUT_COMPACT	1

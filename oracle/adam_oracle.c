@@ -241,6 +241,30 @@ double oracle_sumsq(const void *g, int grad_type, int64_t n, const oracle_seg *s
 		segs = &whole;
 		nsegs = 1;
 	}
+	if (grad_type == ORACLE_FP8) {
+		/*
+		** FP8 gradients (no counterpart in the reference): the norm is defined in its
+		** factored form, SUM_t (scale_t * grad_scale)^2 * SUM_i decode(q_i)^2.  The square of
+		** an E4M3 value is exact in float and the inner sum is exact in double (multiples of
+		** 2^-18 below 2^53), so its order does not matter; only the per-tensor products round.
+		*/
+		for (s = 0; s < nsegs; s++) {
+			const uint8_t *q = (const uint8_t *)g + segs[s].off;
+			const double sc = (double)segs[s].gscale * grad_scale;
+			double inner = 0.0;
+			int64_t i;
+
+#pragma omp parallel for num_threads(threads > 1 ? threads : 1) reduction(+:inner) \
+    if (threads > 1 && segs[s].n > 65536)
+			for (i = 0; i < segs[s].n; i++) {
+				const float d = oracle_fp8_decode(q[i]);
+
+				inner += (double)(d * d);
+			}
+			total += (sc * sc) * inner;
+		}
+		return total;
+	}
 	if (threads <= 1) {
 		/* One accumulator carried through every tensor in slot order: the reference's loop. */
 		for (s = 0; s < nsegs; s++)

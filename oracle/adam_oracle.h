@@ -82,7 +82,10 @@ int	oracle_adam_step_scaled(oracle_adam *o, float *p, void *g, void *m, void *v,
 		uint16_t *twin, const oracle_seg *segs, int nsegs, double lr,
 		double grad_scale, const double *sumsq_override, int threads);
 
-/* Sum over the flat of (g*grad_scale)^2 as the clip block computes it. */
+/*
+** Sum over the flat of (g*grad_scale)^2 as the clip block computes it.  FP8 gradients use the
+** factored form SUM_t (scale_t*grad_scale)^2 * SUM_i decode(q_i)^2 (defined here, unpinned).
+*/
 double	oracle_sumsq(const void *g, int grad_type, int64_t n, const oracle_seg *segs,
 		int nsegs, double grad_scale, int threads);
 

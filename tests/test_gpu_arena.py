@@ -90,11 +90,12 @@ def run_fp32_case(gpu, oracle, tensors, steps, clip, wd, gmul, grad_scale=1.0, s
 
 
 def test_spread_layout_gives_the_same_results(gpu, oracle):
-    """Every flat in its own 16 GiB region of device memory (one 80 GiB allocation)."""
+    """Every flat in its own 16 GiB region of device memory (one 96 GiB allocation)."""
     from anni_amd import lib
     opt = make(gpu, RAGGED, layout=lib.LAYOUT_SPREAD, grad_slots=2)
     assert opt.spread and opt.grad_slot(1) - opt.grad_slot(0) >= 4 * opt.n
     assert opt.o.d_m - opt.o.d_param == 16 << 30 and opt.o.d_v - opt.o.d_m == 16 << 30
+    assert opt.o.d_param_bf16 - opt.o.d_param == 64 << 30 and opt.grad_slot(0) - opt.o.d_param == 80 << 30
     assert opt.grad_slot(2) is None
     opt.free()
     n = sum(t[0] for t in RAGGED)
