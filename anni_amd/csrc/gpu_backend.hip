@@ -272,12 +272,101 @@ void gpu_op_prof_dump(void)
 
 /* ---- memory --------------------------------------------------------------- */
 
+/*
+** Large blocks are spread over device memory.  lang/lm_adam.c asks for its five flats one
+** gpu_malloc at a time (d_param, d_grad, d_param_bf16, later d_m, d_v: lm_adam.c:222-229,
+** 295-297); packed next to each other they would share 16 GiB regions of device memory,
+** which costs the update ~20 % of its bandwidth on MI355X.  So the first large request
+** reserves one slab of six regions (4-region block + 2-region block) and every request of
+** kSpreadMin bytes or more gets a region of its own, in the order 0, 5, 4, 1, 2, 3 -- which
+** puts the caller's p, g, twin, m, v where the arena of anni_adam_create puts them (three
+** flats per 64 GiB group).  Anything that does not fit (no free region, larger than a
+** region, slab not available) is a plain hipMalloc.  ANNI_MALLOC_SPREAD=0 switches it off.
+*/
+static const size_t kSpreadMin = (size_t)256 << 20;
+static const size_t kRegion = (size_t)16 << 30;
+static const int kSpreadRegions = 6;
+static const int kSpreadOrder[kSpreadRegions] = { 0, 5, 4, 1, 2, 3 };
+static char *g_slab;
+static bool g_slab_tried;
+static bool g_region_used[kSpreadRegions];
+static int g_regions_live;
+
+static bool spread_on(void)
+{
+	static int on = -1;
+
+	if (on < 0) {
+		const char *e = getenv("ANNI_MALLOC_SPREAD");
+
+		on = (e && e[0] == '0') ? 0 : 1;
+	}
+	return on == 1;
+}
+
+/* Called with g_mu held.  Returns a region of the slab or nullptr. */
+static void *spread_take(size_t nbytes)
+{
+	if (!spread_on() || nbytes < kSpreadMin || nbytes > kRegion)
+		return nullptr;
+	if (!g_slab && !g_slab_tried) {
+		size_t free_b = 0, total_b = 0;
+		void *p = nullptr;
+
+		g_slab_tried = true;
+		if (hipMemGetInfo(&free_b, &total_b) == hipSuccess
+		    && (size_t)kSpreadRegions * kRegion <= free_b / 2
+		    && hipMalloc(&p, (size_t)kSpreadRegions * kRegion) == hipSuccess)
+			g_slab = (char *)p;
+		(void)hipGetLastError();
+	}
+	if (!g_slab)
+		return nullptr;
+	for (int k = 0; k < kSpreadRegions; k++) {
+		const int r = kSpreadOrder[k];
+
+		if (!g_region_used[r]) {
+			g_region_used[r] = true;
+			g_regions_live++;
+			return g_slab + (size_t)r * kRegion;
+		}
+	}
+	return nullptr;
+}
+
+/* Called with g_mu held.  True when p was a region of the slab (now released). */
+static bool spread_give(void *p)
+{
+	if (!g_slab || (char *)p < g_slab || (char *)p >= g_slab + (size_t)kSpreadRegions * kRegion)
+		return false;
+	const size_t off = (size_t)((char *)p - g_slab);
+
+	if (off % kRegion != 0 || !g_region_used[off / kRegion])
+		return false;
+	g_region_used[off / kRegion] = false;
+	if (--g_regions_live == 0) {
+		/* Last region returned: give the slab back and start over on the next large request. */
+		(void)hipStreamSynchronize(g_stream);
+		(void)hipFree(g_slab);
+		g_slab = nullptr;
+		g_slab_tried = false;
+	}
+	return true;
+}
+
 void *gpu_malloc(size_t nbytes)
 {
 	void *p = nullptr;
 
 	if (nbytes == 0 || !device_ready())
 		return nullptr;
+	{
+		std::lock_guard<std::mutex> lk(g_mu);
+
+		p = spread_take(nbytes);
+	}
+	if (p)
+		return p;
 	if (!hip_ok(hipMalloc(&p, nbytes), "hipMalloc")) {
 		(void)hipGetLastError();
 		return nullptr;
@@ -298,6 +387,8 @@ void gpu_free(void *p)
 			g_twin_fp32 = nullptr;
 			g_twin_n = 0;
 		}
+		if (spread_give(p))
+			return;
 	}
 	(void)hip_ok(hipFree(p), "hipFree");
 }

@@ -351,3 +351,29 @@ def test_the_unchanged_reference_caller_on_this_backend(gpu, oracle):
     R.close()
     gpu.gpu_set_compute_prec(0)
     gpu.gpu_adam_set_weight_decay(0.0)
+
+
+def test_large_allocations_are_spread_over_regions(gpu):
+    """gpu_malloc gives every large block a 16 GiB region of its own, in the order that puts the
+    caller's p, g, twin, m, v (lm_adam.c:222-229,295-297) three to a 64 GiB group."""
+    n = 160 * 1000 * 1000                                # every block >= 256 MiB
+    sizes = [4 * n, 4 * n, 2 * n, 4 * n, 4 * n]
+    ptrs = [gpu.gpu_malloc(sz) for sz in sizes]
+    assert all(ptrs)
+    base = ptrs[0]
+    assert [(p - base) >> 34 for p in ptrs] == [0, 5, 4, 1, 2]
+    assert all((p - base) % (1 << 34) == 0 for p in ptrs)
+    small = gpu.gpu_malloc(1 << 20)                      # small blocks are ordinary allocations
+    assert small and not (base <= small < base + (6 << 34))
+    gpu.gpu_free(ptrs[1])
+    again = gpu.gpu_malloc(4 * n)                        # a freed region is reused
+    assert again == ptrs[1]
+    # the memory is usable: fill and read back the ends of one block
+    assert gpu.gpu_memset(ptrs[3], 0x5a, 4 * n) == 0
+    tail = np.zeros(16, np.uint8)
+    assert gpu.gpu_memcpy_d2h(tail.ctypes.data, ptrs[3] + 4 * n - 16, 16) == 0 and (tail == 0x5a).all()
+    for p in [ptrs[0], again, ptrs[2], ptrs[3], ptrs[4], small]:
+        gpu.gpu_free(p)
+    fresh = gpu.gpu_malloc(4 * n)                        # everything returned: a new slab next time
+    assert fresh
+    gpu.gpu_free(fresh)
