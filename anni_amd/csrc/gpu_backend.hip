@@ -49,8 +49,13 @@ bool device_ready(void)
 	return g_ready;
 }
 
+static void batch_flush(void);
+static int g_batch_dir;
+
 hipStream_t compute_stream(void)
 {
+	if (g_batch_dir != 0)
+		batch_flush();		/* pending small copies go first (see "small copies, batched") */
 	return g_stream;
 }
 
@@ -67,6 +72,175 @@ bool hip_ok(hipError_t err, const char *what)
 	if (!g_err[0])
 		snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(err));
 	return false;
+}
+
+/* ---- small copies, batched ------------------------------------------------- */
+
+/*
+** lang/lm_adam.c moves every bias / LayerNorm vector with its own gpu_memcpy_h2d before the
+** step and its own gpu_memcpy_d2h_async after it (lm_adam.c:372-377,407-413): 146 + 73 copies
+** of a few KiB per step at the reference's 185M size, more time than the two kernels.  Copies
+** of kSmallCopy bytes or less are therefore batched: an H2D is copied into a page-locked
+** staging ring at once (the caller may reuse its buffer on return, as with a pageable
+** cudaMemcpyAsync) and described in a table; the next operation on the stream first launches
+** ONE kernel that moves the whole batch.  A small async D2H is gathered the same way into the
+** ring and handed to its host destination at the next synchronisation, which is when the
+** contract makes it visible (num/gpu.h:44-47).  Order on the stream is kept because every
+** entry point flushes the pending batch before it enqueues anything.
+** ANNI_SMALL_COPY_BATCH=0 switches the batching off.
+*/
+struct CopyDesc {
+	void		*dev;
+	unsigned long long	stage_off;
+	unsigned long long	nbytes;
+};
+
+static const size_t kSmallCopy = (size_t)64 << 10;
+static const size_t kStageBytes = (size_t)16 << 20;
+static const int kDescSlots = 8192;
+static char *g_stage;			/* page-locked, device-visible */
+static CopyDesc *g_desc;		/* page-locked, device-visible */
+static size_t g_stage_used;		/* bump pointers; reset after every full synchronisation */
+static int g_desc_used;
+static int g_batch_first;		/* descriptors [g_batch_first, g_desc_used) are not launched yet */
+/* g_batch_dir (declared above): 0 none, 1 host-to-device, 2 device-to-host */
+struct Delivery {
+	void	*host;
+	size_t	stage_off;
+	size_t	nbytes;
+};
+static Delivery g_deliver[kDescSlots];	/* gathered D2H data waiting for a synchronisation */
+static int g_deliver_n;
+
+__global__ __launch_bounds__(256) void small_copy_kernel(const CopyDesc *desc, char *stage,
+	int to_device)
+{
+	const CopyDesc d = desc[blockIdx.x];
+	char *dev = (char *)d.dev;
+	char *stg = stage + d.stage_off;
+
+	/* byte-wise: sizes and addresses are arbitrary, the batch is a few MiB at most */
+	if (to_device) {
+		for (size_t i = threadIdx.x; i < d.nbytes; i += 256)
+			dev[i] = stg[i];
+	} else {
+		for (size_t i = threadIdx.x; i < d.nbytes; i += 256)
+			stg[i] = dev[i];
+	}
+}
+
+static bool batch_on(void)
+{
+	static int on = -1;
+
+	if (on < 0) {
+		const char *e = getenv("ANNI_SMALL_COPY_BATCH");
+
+		on = (e && e[0] == '0') ? 0 : 1;
+		if (on) {
+			void *a = nullptr, *b = nullptr;
+
+			if (hipHostMalloc(&a, kStageBytes, hipHostMallocDefault) != hipSuccess
+			    || hipHostMalloc(&b, sizeof(CopyDesc) * kDescSlots, hipHostMallocDefault)
+			    != hipSuccess) {
+				(void)hipGetLastError();
+				on = 0;
+			} else {
+				g_stage = (char *)a;
+				g_desc = (CopyDesc *)b;
+			}
+		}
+	}
+	return on == 1;
+}
+
+/* Launches the pending batch.  g_mu held. */
+static void batch_flush_locked(void)
+{
+	const int count = g_desc_used - g_batch_first;
+
+	if (count > 0) {
+		hipLaunchKernelGGL(small_copy_kernel, dim3(count), dim3(256), 0, g_stream,
+		    g_desc + g_batch_first, g_stage, g_batch_dir == 1 ? 1 : 0);
+		(void)hip_ok(hipGetLastError(), "small copy batch");
+	}
+	g_batch_first = g_desc_used;
+	g_batch_dir = 0;
+}
+
+/* After the stream has drained: hand gathered data to its host destinations, recycle the rings.  g_mu held. */
+static void batch_deliver_locked(void)
+{
+	for (int i = 0; i < g_deliver_n; i++)
+		memcpy(g_deliver[i].host, g_stage + g_deliver[i].stage_off, g_deliver[i].nbytes);
+	g_deliver_n = 0;
+	g_stage_used = 0;
+	g_desc_used = 0;
+	g_batch_first = 0;
+}
+
+/* Queues one small copy; false = does not qualify (the caller copies the ordinary way).  g_mu held. */
+static bool batch_add_locked(int dir, void *dev, void *host, size_t nbytes)
+{
+	const size_t need = (nbytes + 255) / 256 * 256;
+
+	if (nbytes > kSmallCopy || !batch_on())
+		return false;
+	if (g_batch_dir != 0 && g_batch_dir != dir)
+		batch_flush_locked();
+	if (g_stage_used + need > kStageBytes || g_desc_used == kDescSlots
+	    || g_deliver_n == kDescSlots) {
+		/* rings full: drain everything, then start over */
+		batch_flush_locked();
+		if (hipStreamSynchronize(g_stream) != hipSuccess)
+			return false;
+		batch_deliver_locked();
+	}
+	g_desc[g_desc_used].dev = dev;
+	g_desc[g_desc_used].stage_off = g_stage_used;
+	g_desc[g_desc_used].nbytes = nbytes;
+	if (dir == 1) {
+		memcpy(g_stage + g_stage_used, host, nbytes);
+	} else {
+		g_deliver[g_deliver_n].host = host;
+		g_deliver[g_deliver_n].stage_off = g_stage_used;
+		g_deliver[g_deliver_n].nbytes = nbytes;
+		g_deliver_n++;
+	}
+	g_desc_used++;
+	g_stage_used += need;
+	g_batch_dir = dir;
+	return true;
+}
+
+static void batch_flush(void)
+{
+	std::lock_guard<std::mutex> lk(g_mu);
+
+	batch_flush_locked();
+}
+
+/* The stream, after the pending small copies have been put on it. */
+static hipStream_t stream_for_op(void)
+{
+	if (g_batch_dir != 0)
+		batch_flush();
+	return g_stream;
+}
+
+/* Waits for the stream and completes the batched D2H copies. */
+static hipError_t sync_stream_and_deliver(void)
+{
+	hipError_t err;
+
+	batch_flush();
+	err = hipStreamSynchronize(g_stream);
+	if (err == hipSuccess) {
+		std::lock_guard<std::mutex> lk(g_mu);
+
+		batch_deliver_locked();
+	}
+	return err;
 }
 
 /* ---- state of the flat drop-in path ------------------------------------- */
@@ -214,7 +388,13 @@ void gpu_device_sync(void)
 
 	if (!device_ready())
 		return;
+	batch_flush();
 	err = hipDeviceSynchronize();
+	if (err == hipSuccess) {
+		std::lock_guard<std::mutex> lk(g_mu);
+
+		batch_deliver_locked();
+	}
 	if (err != hipSuccess) {
 		fprintf(stderr, "gpu_device_sync: %s\n", hipGetErrorString(err));
 		(void)hip_ok(err, "hipDeviceSynchronize");
@@ -228,7 +408,7 @@ int gpu_stream_sync(void)
 {
 	if (!device_ready())
 		return -1;
-	return hip_ok(hipStreamSynchronize(g_stream), "hipStreamSynchronize") ? 0 : -1;
+	return hip_ok(sync_stream_and_deliver(), "hipStreamSynchronize") ? 0 : -1;
 }
 
 void gpu_set_compute_prec(int prec)
@@ -378,6 +558,7 @@ void gpu_free(void *p)
 {
 	if (!p || !device_ready())
 		return;
+	batch_flush();		/* nothing pending may still point into the block */
 	{
 		std::lock_guard<std::mutex> lk(g_mu);
 
@@ -397,7 +578,13 @@ int gpu_memcpy_h2d(void *dst, const void *src, size_t nbytes)
 {
 	if (!dst || !src || nbytes == 0 || !device_ready())
 		return -1;
-	return hip_ok(hipMemcpyAsync(dst, src, nbytes, hipMemcpyHostToDevice, g_stream),
+	if (nbytes <= kSmallCopy) {
+		std::lock_guard<std::mutex> lk(g_mu);
+
+		if (batch_add_locked(1, dst, const_cast<void *>(src), nbytes))
+			return 0;
+	}
+	return hip_ok(hipMemcpyAsync(dst, src, nbytes, hipMemcpyHostToDevice, stream_for_op()),
 	    "h2d") ? 0 : -1;
 }
 
@@ -405,9 +592,9 @@ int gpu_memcpy_d2h(void *dst, const void *src, size_t nbytes)
 {
 	if (!dst || !src || nbytes == 0 || !device_ready())
 		return -1;
-	if (!hip_ok(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, g_stream), "d2h"))
+	if (!hip_ok(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, stream_for_op()), "d2h"))
 		return -1;
-	return hip_ok(hipStreamSynchronize(g_stream), "d2h sync") ? 0 : -1;
+	return hip_ok(sync_stream_and_deliver(), "d2h sync") ? 0 : -1;
 }
 
 /*
@@ -446,7 +633,13 @@ int gpu_memcpy_d2h_async(void *dst, const void *src, size_t nbytes)
 {
 	if (!dst || !src || nbytes == 0 || !device_ready())
 		return -1;
-	return hip_ok(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, g_stream),
+	if (nbytes <= kSmallCopy) {
+		std::lock_guard<std::mutex> lk(g_mu);
+
+		if (batch_add_locked(2, const_cast<void *>(src), dst, nbytes))
+			return 0;
+	}
+	return hip_ok(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, stream_for_op()),
 	    "d2h async") ? 0 : -1;
 }
 
@@ -454,7 +647,7 @@ int gpu_memcpy_d2d(void *dst, const void *src, size_t nbytes)
 {
 	if (!dst || !src || nbytes == 0 || !device_ready())
 		return -1;
-	return hip_ok(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToDevice, g_stream),
+	return hip_ok(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToDevice, stream_for_op()),
 	    "d2d") ? 0 : -1;
 }
 
@@ -462,7 +655,7 @@ int gpu_memset(void *dst, int value, size_t nbytes)
 {
 	if (!dst || nbytes == 0 || !device_ready())
 		return -1;
-	return launch_fill_bytes(g_stream, dst, value, nbytes);
+	return launch_fill_bytes(stream_for_op(), dst, value, nbytes);
 }
 
 void *gpu_host_alloc(size_t nbytes)
@@ -499,7 +692,7 @@ int gpu_adam_seed_bf16_flat(void *bf16, const ann_real *fp32, int n)
 {
 	if (!bf16 || !fp32 || n <= 0 || !device_ready())
 		return -1;
-	return launch_f32_to_bf16(g_stream, (uint16_t *)bf16, fp32, n);
+	return launch_f32_to_bf16(stream_for_op(), (uint16_t *)bf16, fp32, n);
 }
 
 void gpu_half_wt_invalidate(const ann_real *fp32_dev)
@@ -533,6 +726,7 @@ int gpu_grad_sumsq(const ann_real *d_x, int n, double *out)
 	f.g = (void *)d_x;
 	f.n = n;
 	f.grad_type = kF32;
+	(void)stream_for_op();
 	{
 		ProfScope prof(0);
 
@@ -542,7 +736,7 @@ int gpu_grad_sumsq(const ann_real *d_x, int n, double *out)
 	}
 	if (!hip_ok(hipMemcpyAsync(g_host_result, &g_state->sumsq, sizeof(double),
 	    hipMemcpyDeviceToHost, g_stream), "sumsq d2h")
-	    || !hip_ok(hipStreamSynchronize(g_stream), "sumsq sync"))
+	    || !hip_ok(sync_stream_and_deliver(), "sumsq sync"))
 		return -1;
 	*out = *g_host_result;
 	return 0;
@@ -585,6 +779,7 @@ int gpu_adam_step_dev_bf16(ann_real *d_param, void *d_param_bf16, ann_real *d_gr
 	f.moment_type = kF32;
 	f.uniform_flags = (g_wd > 0.0 ? kSegDecay : 0u) | (f.twin ? kSegTwin : 0u);
 	memset(&norm, 0, sizeof(norm));
+	(void)stream_for_op();
 	ProfScope prof(1);
 
 	return launch_update(g_stream, f, c, grad_scale, norm);

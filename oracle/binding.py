@@ -266,8 +266,78 @@ def ref_hip():
         R.ref_adam_release_device.argtypes = [C.c_void_p]
         R.ref_adam_export.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         R.ref_adam_free.argtypes = [C.c_void_p]
+        R.ref_model_create.argtypes = [C.c_int, C.c_double, C.c_double, C.c_double]
+        R.ref_model_create.restype = C.c_void_p
+        R.ref_model_n.argtypes = [C.c_void_p]
+        R.ref_model_n.restype = C.c_long
+        for f in ("ref_model_n_segs", "ref_model_t", "ref_model_on_device"):
+            getattr(R, f).argtypes = [C.c_void_p]
+            getattr(R, f).restype = C.c_int
+        R.ref_model_last_norm.argtypes = [C.c_void_p]
+        R.ref_model_last_norm.restype = C.c_double
+        R.ref_model_seg.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_long), C.POINTER(C.c_long),
+                                    C.POINTER(C.c_int)]
+        R.ref_model_get_params.argtypes = [C.c_void_p, C.c_void_p]
+        R.ref_model_get_moments.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        R.ref_model_set_grads.argtypes = [C.c_void_p, C.c_void_p]
+        R.ref_model_set_grads.restype = C.c_int
+        R.ref_model_step.argtypes = [C.c_void_p, C.c_double, C.c_double]
+        R.ref_model_step.restype = C.c_int
+        R.ref_model_free.argtypes = [C.c_void_p]
         _ref_hip = R
     return _ref_hip
+
+
+class RefModelOnBackend:
+    """The reference's real lm + lm_adam_create (its compile-time 185M sizes) on libanni_gpu_hip.so."""
+
+    def __init__(self, vocab=16384, beta2=0.95, weight_decay=0.1, grad_clip=1.0):
+        self.R = ref_hip()
+        self.h = self.R.ref_model_create(vocab, beta2, weight_decay, grad_clip)
+        if not self.h:
+            raise MemoryError("ref_model_create")
+        self.n = self.R.ref_model_n(self.h)
+        self.n_segs = self.R.ref_model_n_segs(self.h)
+
+    def segs(self):
+        out = []
+        off, n, im = C.c_long(0), C.c_long(0), C.c_int(0)
+        for i in range(self.n_segs):
+            self.R.ref_model_seg(self.h, i, C.byref(off), C.byref(n), C.byref(im))
+            out.append((off.value, n.value, bool(im.value)))
+        return out
+
+    def params(self):
+        p = np.empty(self.n, np.float32)
+        self.R.ref_model_get_params(self.h, _ptr(p))
+        return p
+
+    def moments(self):
+        m = np.empty(self.n, np.float32)
+        v = np.empty(self.n, np.float32)
+        self.R.ref_model_get_moments(self.h, _ptr(m), _ptr(v))
+        return m, v
+
+    def set_grads(self, g):
+        assert g.dtype == np.float32 and g.size == self.n
+        if self.R.ref_model_set_grads(self.h, _ptr(g)) != 0:
+            raise RuntimeError("ref_model_set_grads")
+
+    def step(self, lr, grad_scale=1.0):
+        return self.R.ref_model_step(self.h, lr, grad_scale)
+
+    @property
+    def on_device(self):
+        return bool(self.R.ref_model_on_device(self.h))
+
+    @property
+    def last_grad_norm(self):
+        return self.R.ref_model_last_norm(self.h)
+
+    def close(self):
+        if self.h:
+            self.R.ref_model_free(self.h)
+            self.h = None
 
 
 class RefAdamOnBackend:

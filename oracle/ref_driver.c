@@ -145,6 +145,108 @@ void ref_adam_free(ref_adam *r)
 	free(r);
 }
 
+/*
+** The production flow: a real lm (the reference's compile-time sizes: D=1024, 16 heads, FF
+** 4096, 12 blocks, lang/lm_config.h:8-24; untied embedding) and lm_adam_create over it
+** (lang/lm_adam.c:79-139).  With a real backend linked, lm_adam_step_scaled aliases every
+** weight / gradient matrix into its flats and keeps bias / LayerNorm vectors on the host,
+** exactly as in training.
+*/
+typedef struct ref_model {
+	lm	*model;
+	lm_adam	*opt;
+} ref_model;
+
+ref_model *ref_model_create(int vocab, double beta2, double wd, double clip)
+{
+	ref_model *r = calloc(1, sizeof(*r));
+
+	if (!r)
+		return NULL;
+	r->model = lm_create_vocab(vocab);
+	if (r->model)
+		r->opt = lm_adam_create(r->model);
+	if (!r->opt) {
+		lm_free(&r->model);
+		free(r);
+		return NULL;
+	}
+	r->opt->beta2 = beta2;
+	r->opt->weight_decay = wd;
+	r->opt->grad_clip = clip;
+	return r;
+}
+
+long ref_model_n(const ref_model *r) { return r->opt->n; }
+int ref_model_n_segs(const ref_model *r) { return r->opt->n_segs; }
+int ref_model_t(const ref_model *r) { return r->opt->t; }
+int ref_model_on_device(const ref_model *r) { return r->opt->d_param != NULL; }
+double ref_model_last_norm(const ref_model *r) { return r->opt->last_grad_norm; }
+
+/* seg i: off, n, 1 for a matrix / 0 for a vector. */
+void ref_model_seg(const ref_model *r, int i, long *off, long *n, int *is_mat)
+{
+	*off = r->opt->segs[i].off;
+	*n = r->opt->segs[i].n;
+	*is_mat = r->opt->segs[i].w != NULL;
+}
+
+/* Parameters (host view) into / out of one flat array in slot order. */
+void ref_model_get_params(ref_model *r, float *flat)
+{
+	long i;
+
+	lm_adam_sync_host(r->opt);	/* device-authoritative weights and m/v -> host */
+	for (i = 0; i < r->opt->n; i++)
+		flat[i] = *r->opt->slots[i].param;
+}
+
+void ref_model_get_moments(ref_model *r, float *m, float *v)
+{
+	long i;
+
+	lm_adam_sync_host(r->opt);
+	for (i = 0; i < r->opt->n; i++) {
+		m[i] = r->opt->slots[i].m;
+		v[i] = r->opt->slots[i].v;
+	}
+}
+
+/*
+** New gradients from one flat array: host dW / db everywhere (what the first step and the
+** vector segments read), and straight into the device flat once the matrices are aliased
+** there (where backward would have written them).
+*/
+int ref_model_set_grads(ref_model *r, const float *flat)
+{
+	long i;
+
+	for (i = 0; i < r->opt->n; i++)
+		*r->opt->slots[i].grad = flat[i];
+	/* host writes leave a mat host-authoritative (num/mat.h: mat_host_dirty) unless it is aliased */
+	for (i = 0; i < r->opt->n_segs; i++)
+		if (r->opt->segs[i].dw && r->opt->segs[i].dw->on_device != MAT_DEV_ALIASED)
+			mat_host_dirty(r->opt->segs[i].dw);
+	if (r->opt->d_grad)
+		return gpu_memcpy_h2d(r->opt->d_grad, flat, (size_t)r->opt->n * sizeof(float));
+	return 0;
+}
+
+int ref_model_step(ref_model *r, double lr, double grad_scale)
+{
+	lm_adam_step_scaled(r->opt, lr, grad_scale);
+	return r->opt->t;
+}
+
+void ref_model_free(ref_model *r)
+{
+	if (!r)
+		return;
+	lm_adam_free(&r->opt);
+	lm_free(&r->model);
+	free(r);
+}
+
 double ref_step_lr(double base_lr, int step, int warmup, int decay_steps,
 	const char *kind, int sched_from)
 {

@@ -377,3 +377,47 @@ def test_large_allocations_are_spread_over_regions(gpu):
     fresh = gpu.gpu_malloc(4 * n)                        # everything returned: a new slab next time
     assert fresh
     gpu.gpu_free(fresh)
+
+
+def test_small_copies_are_batched_in_order(gpu):
+    """Small gpu_memcpy_h2d / gpu_memcpy_d2h_async calls (the bias / LayerNorm traffic of
+    lm_adam.c:372-377,407-413) go through the staging rings: contents, ordering against other
+    stream work, reuse of the caller's buffer after return, and ring overflow."""
+    from anni_amd.lm_adam import DeviceBuffer
+    rng = np.random.default_rng(3)
+    nseg, seg = 500, 40000                               # 500 x 40 kB = 20 MB: overflows the 16 MiB ring
+    d = DeviceBuffer(nseg * seg)
+    assert gpu.gpu_memset(d.ptr, 0xee, nseg * seg) == 0
+    want = np.empty(nseg * seg, np.uint8)
+    scratch = np.empty(seg, np.uint8)
+    for i in range(nseg):
+        scratch[:] = rng.integers(0, 255, seg, dtype=np.uint8)
+        want[i * seg:(i + 1) * seg] = scratch
+        assert gpu.gpu_memcpy_h2d(d.ptr + i * seg, scratch.ctypes.data, seg) == 0
+        scratch[:] = 0                                   # the caller may reuse its buffer at once
+    assert (d.download(np.uint8, nseg * seg) == want).all()
+    # h2d batch, then a fill of part of it, then more h2d: order on the stream is kept
+    a = np.full(1000, 7, np.uint8)
+    assert gpu.gpu_memcpy_h2d(d.ptr, a.ctypes.data, 1000) == 0
+    assert gpu.gpu_memset(d.ptr + 500, 9, 1000) == 0
+    b = np.full(100, 3, np.uint8)
+    assert gpu.gpu_memcpy_h2d(d.ptr + 1400, b.ctypes.data, 100) == 0
+    got = d.download(np.uint8, 2000)
+    assert (got[:500] == 7).all() and (got[500:1400] == 9).all() and (got[1400:1500] == 3).all()
+    assert (got[1500:] == want[1500:2000]).all()
+    # async d2h of many pieces, visible after the stream sync; odd sizes and offsets
+    outs = []
+    for i in range(200):
+        off, ln = 12345 * i + (i % 7), 1 + (i * 37) % 5000
+        o = np.zeros(ln, np.uint8)
+        assert gpu.gpu_memcpy_d2h_async(o.ctypes.data, d.ptr + off, ln) == 0
+        outs.append((off, ln, o))
+    assert gpu.gpu_memset(d.ptr, 0, nseg * seg) == 0     # later work must not reach the copies
+    assert gpu.gpu_stream_sync() == 0
+    ref = want.copy()
+    ref[:500] = 7
+    ref[500:1400] = 9
+    ref[1400:1500] = 3
+    for off, ln, o in outs:
+        assert (o == ref[off:off + ln]).all(), (off, ln)
+    assert not d.download(np.uint8, 4096).any()

@@ -220,3 +220,46 @@ def test_config5_1p4b_fp8_grads_and_nan_skip(gpu, oracle):
     assert not opt.download("grad").any()
     print("1.4b fp8 NaN step skipped, state unchanged", flush=True)
     opt.free()
+
+
+def test_reference_production_flow_on_this_backend(gpu, oracle):
+    """The reference's own lm (its compile-time sizes: 184,676,352 parameters with the untied
+    16384-token embedding, 147 segments) and lm_adam_create, compiled from the reference tree and
+    linked against libanni_gpu_hip.so: lm_adam_step_scaled aliases the matrices into its device
+    flats, keeps the 73 bias / LayerNorm vectors on the host, clips, decays every slot -- the
+    training flow, unchanged.  Four steps, then every parameter and moment against the oracle."""
+    if not oracle.ref_hip_available():
+        pytest.skip("oracle/_ref/libanni_ref_hip.so not built (reference tree absent at build time)")
+    import time
+    gpu.gpu_set_compute_prec(1)
+    M = oracle.RefModelOnBackend(16384, beta2=0.95, weight_decay=0.1, grad_clip=1.0)
+    n = M.n
+    assert n == 184676352 and M.n_segs == 3 + 12 * 12
+    segs = M.segs()
+    assert sum(1 for s in segs if not s[2]) == 1 + 6 * 12 and segs[-1][0] + segs[-1][1] == n
+    P = M.params()
+    Mo, Vo = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, threads=THREADS, simd=oracle.cpu_simd())
+    rng = np.random.default_rng(5)
+    unit = 1.0 / (math.sqrt(n) * 1e-3)
+    for t in range(1, 5):
+        g = rng.standard_normal(n, dtype=np.float32) * np.float32(1e-3)
+        M.set_grads(g)
+        gpu.gpu_device_sync()
+        lr = oracle.lr(3e-4, t - 1, 100, 1000, "cosine")
+        gs = unit * (1.7 if t % 2 else 0.6)
+        t0 = time.perf_counter()
+        assert M.step(lr, gs) == t and M.on_device
+        dt = (time.perf_counter() - t0) * 1e3
+        norm = M.last_grad_norm                      # sqrt(ss) * |gs| (lm_adam.c:472)
+        assert abs(norm - (1.7 if t % 2 else 0.6)) < 5e-3
+        eff = gs * (1.0 / norm) if norm > 1.0 else gs
+        O.step(P, g, Mo, Vo, lr, eff)
+        print("reference lm_adam_step_scaled step %d: %.2f ms wall (norm %.4f)" % (t, dt, norm),
+              flush=True)
+    p = M.params()
+    m, v = M.moments()
+    assert same_bits(p, P) and same_bits(m, Mo) and same_bits(v, Vo)
+    M.close()
+    gpu.gpu_set_compute_prec(0)
+    gpu.gpu_adam_set_weight_decay(0.0)
