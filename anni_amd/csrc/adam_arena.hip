@@ -10,6 +10,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <unistd.h>
 #include <new>
 #include <vector>
 #include "adam_kernels.h"
@@ -648,6 +649,190 @@ int anni_adam_time_steps(anni_adam *opt, int count, void *const *grads, int n_gr
 	for (size_t i = 0; i < ev.size(); i++)
 		(void)hipEventDestroy(ev[i]);
 	return rc;
+}
+
+/* ---- optimizer block of a checkpoint (lang/lm_serialize.c:263-331,526-587) ----------- */
+
+/* Slots per staging round: the reference's ADAM_CHUNK (lm_serialize.c:261), 16 MiB of pairs. */
+static const int64_t kCkptChunk = (int64_t)1 << 21;
+
+/* Two page-locked + two device staging buffers of one chunk each, for the lifetime of one call. */
+struct CkptStage {
+	float	*host[2];
+	float	*dev[2];
+
+	CkptStage() : host{nullptr, nullptr}, dev{nullptr, nullptr} {}
+	bool init(void)
+	{
+		const size_t bytes = (size_t)kCkptChunk * 2 * sizeof(float);
+
+		for (int i = 0; i < 2; i++)
+			if (hipHostMalloc((void **)&host[i], bytes, hipHostMallocDefault) != hipSuccess
+			    || hipMalloc((void **)&dev[i], bytes) != hipSuccess) {
+				(void)hipGetLastError();
+				return false;
+			}
+		return true;
+	}
+	~CkptStage()
+	{
+		for (int i = 0; i < 2; i++) {
+			if (host[i])
+				(void)hipHostFree(host[i]);
+			if (dev[i])
+				(void)hipFree(dev[i]);
+		}
+	}
+};
+
+int anni_adam_export_mv(anni_adam *opt, int64_t first, int64_t count, float *pairs)
+{
+	hipStream_t st;
+	CkptStage sg;
+	int rc = 0;
+
+	if (!opt || !opt->priv || !pairs || first < 0 || count < 0 || first + count > opt->n
+	    || !device_ready())
+		return -1;
+	if (count == 0)
+		return 0;
+	if (!sg.init())
+		return -1;
+	st = compute_stream();
+	for (int64_t at = 0, k = 0; rc == 0; at += kCkptChunk, k++) {
+		const int64_t c = count - at < kCkptChunk ? count - at : kCkptChunk;
+		const int b = (int)(k & 1);
+
+		if (c > 0) {
+			if (launch_mv_interleave(st, sg.dev[b], opt->d_m, opt->d_v, opt->cfg.moment_type,
+			    first + at, c) != 0
+			    || !hip_ok(hipMemcpyAsync(sg.host[b], sg.dev[b], (size_t)c * 2 * sizeof(float),
+			    hipMemcpyDeviceToHost, st), "export_mv d2h"))
+				rc = -1;
+		}
+		if (rc == 0 && !hip_ok(hipStreamSynchronize(st), "export_mv sync"))
+			rc = -1;
+		if (rc == 0 && c > 0)
+			memcpy(pairs + 2 * at, sg.host[b], (size_t)c * 2 * sizeof(float));
+		if (at + kCkptChunk >= count)
+			break;
+	}
+	return rc;
+}
+
+int anni_adam_import_mv(anni_adam *opt, int64_t first, int64_t count, const float *pairs)
+{
+	hipStream_t st;
+	CkptStage sg;
+	int rc = 0;
+
+	if (!opt || !opt->priv || !pairs || first < 0 || count < 0 || first + count > opt->n
+	    || !device_ready())
+		return -1;
+	if (count == 0)
+		return 0;
+	if (!sg.init())
+		return -1;
+	st = compute_stream();
+	for (int64_t at = 0, k = 0; at < count && rc == 0; at += kCkptChunk, k++) {
+		const int64_t c = count - at < kCkptChunk ? count - at : kCkptChunk;
+		const int b = (int)(k & 1);
+
+		/* buffer b was last used two chunks ago: wait before overwriting it */
+		if (k >= 2 && !hip_ok(hipStreamSynchronize(st), "import_mv sync"))
+			rc = -1;
+		if (rc == 0) {
+			memcpy(sg.host[b], pairs + 2 * at, (size_t)c * 2 * sizeof(float));
+			if (!hip_ok(hipMemcpyAsync(sg.dev[b], sg.host[b], (size_t)c * 2 * sizeof(float),
+			    hipMemcpyHostToDevice, st), "import_mv h2d")
+			    || launch_mv_deinterleave(st, opt->d_m, opt->d_v, opt->cfg.moment_type,
+			    sg.dev[b], first + at, c) != 0)
+				rc = -1;
+		}
+	}
+	if (!hip_ok(hipStreamSynchronize(st), "import_mv sync"))
+		rc = -1;
+	return rc;
+}
+
+static int write_all(int fd, const void *buf, size_t n)
+{
+	const char *p = (const char *)buf;
+
+	while (n > 0) {
+		const ssize_t w = write(fd, p, n);
+
+		if (w <= 0)
+			return -1;
+		p += w;
+		n -= (size_t)w;
+	}
+	return 0;
+}
+
+static int read_all(int fd, void *buf, size_t n)
+{
+	char *p = (char *)buf;
+
+	while (n > 0) {
+		const ssize_t r = read(fd, p, n);
+
+		if (r <= 0)
+			return -1;
+		p += r;
+		n -= (size_t)r;
+	}
+	return 0;
+}
+
+int anni_adam_write_state(anni_adam *opt, int fd, int epoch, int step)
+{
+	int32_t head[5];
+	std::vector<float> buf;
+
+	if (!opt || !opt->priv || fd < 0 || opt->n > INT32_MAX)
+		return -1;
+	head[0] = 1;			/* lm_serialize.c:319-321: has_adam, epoch, step, t, n */
+	head[1] = epoch;
+	head[2] = step;
+	head[3] = opt->t;
+	head[4] = (int32_t)opt->n;
+	if (write_all(fd, head, sizeof(head)) != 0)
+		return -1;
+	buf.resize((size_t)kCkptChunk * 2);
+	for (int64_t at = 0; at < opt->n; at += kCkptChunk) {
+		const int64_t c = opt->n - at < kCkptChunk ? opt->n - at : kCkptChunk;
+
+		if (anni_adam_export_mv(opt, at, c, buf.data()) != 0
+		    || write_all(fd, buf.data(), (size_t)c * 2 * sizeof(float)) != 0)
+			return -1;
+	}
+	return 0;
+}
+
+int anni_adam_read_state(anni_adam *opt, int fd, int *epoch, int *step)
+{
+	int32_t head[5];
+	std::vector<float> buf;
+
+	if (!opt || !opt->priv || fd < 0)
+		return -1;
+	if (read_all(fd, head, sizeof(head)) != 0 || head[0] != 1 || head[4] != opt->n)
+		return -1;		/* lm_serialize.c:546-562: has_adam == 1 and the same slot count */
+	buf.resize((size_t)kCkptChunk * 2);
+	for (int64_t at = 0; at < opt->n; at += kCkptChunk) {
+		const int64_t c = opt->n - at < kCkptChunk ? opt->n - at : kCkptChunk;
+
+		if (read_all(fd, buf.data(), (size_t)c * 2 * sizeof(float)) != 0
+		    || anni_adam_import_mv(opt, at, c, buf.data()) != 0)
+			return -1;
+	}
+	opt->t = head[3];		/* so the learning-rate schedule continues (lm_serialize.c:564) */
+	if (epoch)
+		*epoch = head[1];
+	if (step)
+		*step = head[2];
+	return 0;
 }
 
 /* ---- learning-rate schedule (lang/lm_train.c:98-124,398-411) ------------------ */

@@ -88,6 +88,12 @@ int	launch_finalize(hipStream_t st, const double *partials, int n_partials, doub
 int	launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double grad_scale,
 		const NormIn &norm);
 int	launch_f32_to_bf16(hipStream_t st, uint16_t *dst, const float *src, int64_t n);
+/* pairs[2k] = m[first+k], pairs[2k+1] = v[first+k] as floats (bf16 moments widen exactly). */
+int	launch_mv_interleave(hipStream_t st, float *pairs, const void *m, const void *v,
+		int moment_type, int64_t first, int64_t count);
+/* The inverse: m[first+k] = pairs[2k], v[first+k] = pairs[2k+1] (bf16 moments: round to nearest even). */
+int	launch_mv_deinterleave(hipStream_t st, void *m, void *v, int moment_type, const float *pairs,
+		int64_t first, int64_t count);
 int	launch_fill_bytes(hipStream_t st, void *dst, int value, size_t nbytes);
 
 } /* namespace anni */

@@ -516,6 +516,41 @@ __global__ __launch_bounds__(kThreads) void f32_to_bf16_kernel(uint16_t *dst,
 		dst[i] = (uint16_t)bf16_rne(src[i]);
 }
 
+/*
+** Checkpoint layout of the moments: per slot one (m, v) float pair (lang/lm_serialize.c:263-296).
+** A lane handles one slot: two scalar loads, one 8-byte store (or the reverse).
+*/
+template <int MT>
+__global__ __launch_bounds__(kThreads) void mv_interleave_kernel(float *pairs, const void *m,
+	const void *v, int64_t first, int64_t count)
+{
+	typedef float f32x2 __attribute__((ext_vector_type(2)));
+	const int64_t stride = (int64_t)gridDim.x * kThreads;
+
+	for (int64_t k = (int64_t)blockIdx.x * kThreads + threadIdx.x; k < count; k += stride) {
+		f32x2 mv;
+
+		mv.x = load_one<MT>(m, first + k, 1.0f);
+		mv.y = load_one<MT>(v, first + k, 1.0f);
+		*(f32x2 *)(pairs + 2 * k) = mv;
+	}
+}
+
+template <int MT>
+__global__ __launch_bounds__(kThreads) void mv_deinterleave_kernel(void *m, void *v,
+	const float *pairs, int64_t first, int64_t count)
+{
+	typedef float f32x2 __attribute__((ext_vector_type(2)));
+	const int64_t stride = (int64_t)gridDim.x * kThreads;
+
+	for (int64_t k = (int64_t)blockIdx.x * kThreads + threadIdx.x; k < count; k += stride) {
+		const f32x2 mv = *(const f32x2 *)(pairs + 2 * k);
+
+		store_one<MT>(m, first + k, mv.x);
+		store_one<MT>(v, first + k, mv.y);
+	}
+}
+
 /* Byte fill on the stream (a kernel, so it can sit in a captured graph). */
 __global__ __launch_bounds__(kThreads) void fill_bytes_kernel(uint8_t *dst, uint32_t pattern,
 	size_t nbytes, size_t head, size_t n16)
@@ -771,6 +806,38 @@ int launch_f32_to_bf16(hipStream_t st, uint16_t *dst, const float *src, int64_t 
 		return -1;
 	hipLaunchKernelGGL(f32_to_bf16_kernel, dim3(helper_grid(n / kQuad + 1)), dim3(kThreads),
 	    0, st, dst, src, n, aligned(src, 16) && aligned(dst, 8) ? 1 : 0);
+	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int launch_mv_interleave(hipStream_t st, float *pairs, const void *m, const void *v,
+	int moment_type, int64_t first, int64_t count)
+{
+	if (!pairs || !m || !v || first < 0 || count <= 0 || !aligned(pairs, 8))
+		return -1;
+	if (moment_type == kF32)
+		hipLaunchKernelGGL((mv_interleave_kernel<kF32>), dim3(helper_grid(count)), dim3(kThreads),
+		    0, st, pairs, m, v, first, count);
+	else if (moment_type == kBF16)
+		hipLaunchKernelGGL((mv_interleave_kernel<kBF16>), dim3(helper_grid(count)),
+		    dim3(kThreads), 0, st, pairs, m, v, first, count);
+	else
+		return -1;
+	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int launch_mv_deinterleave(hipStream_t st, void *m, void *v, int moment_type, const float *pairs,
+	int64_t first, int64_t count)
+{
+	if (!pairs || !m || !v || first < 0 || count <= 0 || !aligned(pairs, 8))
+		return -1;
+	if (moment_type == kF32)
+		hipLaunchKernelGGL((mv_deinterleave_kernel<kF32>), dim3(helper_grid(count)),
+		    dim3(kThreads), 0, st, m, v, pairs, first, count);
+	else if (moment_type == kBF16)
+		hipLaunchKernelGGL((mv_deinterleave_kernel<kBF16>), dim3(helper_grid(count)),
+		    dim3(kThreads), 0, st, m, v, pairs, first, count);
+	else
+		return -1;
 	return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

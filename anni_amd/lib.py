@@ -91,6 +91,11 @@ _PROTOS = {
                                        C.c_int, C.POINTER(C.c_double),
                                        C.POINTER(C.c_double), C.POINTER(C.c_float),
                                        C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+    "anni_adam_export_mv": (C.c_int, [C.POINTER(Adam), C.c_int64, C.c_int64, C.c_void_p]),
+    "anni_adam_import_mv": (C.c_int, [C.POINTER(Adam), C.c_int64, C.c_int64, C.c_void_p]),
+    "anni_adam_write_state": (C.c_int, [C.POINTER(Adam), C.c_int, C.c_int, C.c_int]),
+    "anni_adam_read_state": (C.c_int, [C.POINTER(Adam), C.c_int, C.POINTER(C.c_int),
+                                       C.POINTER(C.c_int)]),
     "anni_lr_set_schedule": (None, [C.c_int, C.c_int, C.c_char_p]),
     "anni_lr_set_sched_from": (None, [C.c_int]),
     "anni_lr_step": (C.c_double, [C.c_double, C.c_int]),

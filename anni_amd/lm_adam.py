@@ -136,6 +136,32 @@ class LmAdam:
         if self.L.anni_adam_bind_grad(self.h, ptr) != 0:
             raise RuntimeError("anni_adam_bind_grad failed")
 
+    # -- the optimizer block of a checkpoint (lang/lm_serialize.c:263-331,526-587) -----------
+    def export_mv(self, first=0, count=None):
+        """(m, v) float pairs of slots [first, first+count) as a (count, 2) array."""
+        count = self.n - first if count is None else count
+        out = np.empty((count, 2), np.float32)
+        if self.L.anni_adam_export_mv(self.h, first, count, out.ctypes.data) != 0:
+            raise RuntimeError("anni_adam_export_mv failed")
+        return out
+
+    def import_mv(self, pairs, first=0):
+        pairs = np.ascontiguousarray(pairs, dtype=np.float32).reshape(-1, 2)
+        if self.L.anni_adam_import_mv(self.h, first, pairs.shape[0], pairs.ctypes.data) != 0:
+            raise RuntimeError("anni_adam_import_mv failed")
+
+    def write_state(self, fd, epoch, step):
+        """has_adam, epoch, step, t, n and the n pairs, as lm_save_checkpoint writes them."""
+        if self.L.anni_adam_write_state(self.h, fd, epoch, step) != 0:
+            raise RuntimeError("anni_adam_write_state failed")
+
+    def read_state(self, fd):
+        """Reads the block lm_load_checkpoint reads; restores t; returns (epoch, step)."""
+        ep, st = C.c_int(-1), C.c_int(-1)
+        if self.L.anni_adam_read_state(self.h, fd, C.byref(ep), C.byref(st)) != 0:
+            raise ValueError("anni_adam_read_state refused the block")
+        return ep.value, st.value
+
     def free(self):
         if getattr(self, "h", None):
             hp = C.POINTER(_l.Adam)(self.h.contents)

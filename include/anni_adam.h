@@ -131,6 +131,19 @@ int	anni_adam_step(anni_adam *opt, double lr);
 /* Waits for the stream and fills last_sumsq / last_grad_norm / last_grad_scale / last_skipped / last_clipped. */
 int	anni_adam_sync_stats(anni_adam *opt);
 
+/*
+** The optimizer block of the reference's checkpoint (lang/lm_serialize.c:263-331,526-587):
+** five int32 {1, epoch, step, t, n} followed by n (m, v) float pairs in slot order, written
+** from / read into the arena through an interleave kernel and page-locked staging in chunks
+** of 2^21 slots.  bf16 moments widen exactly on export and round to nearest even on import.
+** export / import move the pairs of slots [first, first+count) to / from host memory;
+** write / read move the whole block through a file descriptor (read restores t).
+*/
+int	anni_adam_export_mv(anni_adam *opt, int64_t first, int64_t count, float *pairs);
+int	anni_adam_import_mv(anni_adam *opt, int64_t first, int64_t count, const float *pairs);
+int	anni_adam_write_state(anni_adam *opt, int fd, int epoch, int step);
+int	anni_adam_read_state(anni_adam *opt, int fd, int *epoch, int *step);
+
 /* lm_train_step_lr and its setters (lang/lm_train.c:98-124,398-411); kind "none" / "linear" / "cosine". */
 void	anni_lr_set_schedule(int warmup_steps, int decay_steps, const char *kind);
 void	anni_lr_set_sched_from(int from);

@@ -266,38 +266,81 @@ def ref_hip():
         R.ref_adam_release_device.argtypes = [C.c_void_p]
         R.ref_adam_export.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         R.ref_adam_free.argtypes = [C.c_void_p]
-        R.ref_model_create.argtypes = [C.c_int, C.c_double, C.c_double, C.c_double]
-        R.ref_model_create.restype = C.c_void_p
-        R.ref_model_n.argtypes = [C.c_void_p]
-        R.ref_model_n.restype = C.c_long
-        for f in ("ref_model_n_segs", "ref_model_t", "ref_model_on_device"):
-            getattr(R, f).argtypes = [C.c_void_p]
-            getattr(R, f).restype = C.c_int
-        R.ref_model_last_norm.argtypes = [C.c_void_p]
-        R.ref_model_last_norm.restype = C.c_double
-        R.ref_model_seg.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_long), C.POINTER(C.c_long),
-                                    C.POINTER(C.c_int)]
-        R.ref_model_get_params.argtypes = [C.c_void_p, C.c_void_p]
-        R.ref_model_get_moments.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
-        R.ref_model_set_grads.argtypes = [C.c_void_p, C.c_void_p]
-        R.ref_model_set_grads.restype = C.c_int
-        R.ref_model_step.argtypes = [C.c_void_p, C.c_double, C.c_double]
-        R.ref_model_step.restype = C.c_int
-        R.ref_model_free.argtypes = [C.c_void_p]
+        _declare_model(R)
         _ref_hip = R
     return _ref_hip
 
 
-class RefModelOnBackend:
-    """The reference's real lm + lm_adam_create (its compile-time 185M sizes) on libanni_gpu_hip.so."""
+def _declare_model(R):
+    R.ref_model_create.argtypes = [C.c_int, C.c_double, C.c_double, C.c_double]
+    R.ref_model_create.restype = C.c_void_p
+    R.ref_model_n.argtypes = [C.c_void_p]
+    R.ref_model_n.restype = C.c_long
+    for f in ("ref_model_n_segs", "ref_model_t", "ref_model_on_device"):
+        getattr(R, f).argtypes = [C.c_void_p]
+        getattr(R, f).restype = C.c_int
+    R.ref_model_last_norm.argtypes = [C.c_void_p]
+    R.ref_model_last_norm.restype = C.c_double
+    R.ref_model_seg.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_long), C.POINTER(C.c_long),
+                                C.POINTER(C.c_int)]
+    R.ref_model_get_params.argtypes = [C.c_void_p, C.c_void_p]
+    R.ref_model_get_moments.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+    R.ref_model_set_grads.argtypes = [C.c_void_p, C.c_void_p]
+    R.ref_model_set_grads.restype = C.c_int
+    R.ref_model_step.argtypes = [C.c_void_p, C.c_double, C.c_double]
+    R.ref_model_step.restype = C.c_int
+    R.ref_model_save_checkpoint.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_char_p]
+    R.ref_model_save_checkpoint.restype = C.c_int
+    R.ref_model_load_checkpoint.argtypes = [C.c_char_p, C.POINTER(C.c_int), C.POINTER(C.c_int)]
+    R.ref_model_load_checkpoint.restype = C.c_void_p
+    R.ref_model_free.argtypes = [C.c_void_p]
 
-    def __init__(self, vocab=16384, beta2=0.95, weight_decay=0.1, grad_clip=1.0):
-        self.R = ref_hip()
-        self.h = self.R.ref_model_create(vocab, beta2, weight_decay, grad_clip)
+
+_ref_cpu_model = None
+
+
+def ref_cpu_model_lib():
+    """The reference compiled with its own CPU stub backend, model entry points declared."""
+    global _ref_cpu_model
+    if _ref_cpu_model is None:
+        if not os.path.exists(REF_SO):
+            raise FileNotFoundError(REF_SO)
+        R = C.CDLL(REF_SO)
+        _declare_model(R)
+        _ref_cpu_model = R
+    return _ref_cpu_model
+
+
+class RefModelOnBackend:
+    """The reference's real lm + lm_adam_create (its compile-time 185M sizes) on libanni_gpu_hip.so
+    (backend="hip") or on its own CPU stub (backend="cpu")."""
+
+    def __init__(self, vocab=16384, beta2=0.95, weight_decay=0.1, grad_clip=1.0, backend="hip",
+                 _handle=None):
+        self.R = ref_hip() if backend == "hip" else ref_cpu_model_lib()
+        self.h = _handle or self.R.ref_model_create(vocab, beta2, weight_decay, grad_clip)
         if not self.h:
             raise MemoryError("ref_model_create")
         self.n = self.R.ref_model_n(self.h)
         self.n_segs = self.R.ref_model_n_segs(self.h)
+
+    @classmethod
+    def load_checkpoint(cls, path, backend="hip"):
+        """lm_load_checkpoint: returns (model, epoch, step), or raises when the loader refuses the file."""
+        R = ref_hip() if backend == "hip" else ref_cpu_model_lib()
+        ep, st = C.c_int(-1), C.c_int(-1)
+        h = R.ref_model_load_checkpoint(os.fsencode(path), C.byref(ep), C.byref(st))
+        if not h:
+            raise ValueError("lm_load_checkpoint refused " + str(path))
+        return cls(backend=backend, _handle=h), ep.value, st.value
+
+    def save_checkpoint(self, path, epoch, step):
+        if self.R.ref_model_save_checkpoint(self.h, epoch, step, os.fsencode(path)) != 0:
+            raise RuntimeError("lm_save_checkpoint")
+
+    @property
+    def t(self):
+        return self.R.ref_model_t(self.h)
 
     def segs(self):
         out = []

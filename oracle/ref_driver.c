@@ -12,6 +12,7 @@
 #include <string.h>
 #include "gpu.h"
 #include "lm_adam.h"
+#include "lm_serialize.h"
 #include "lm_train.h"
 
 typedef struct ref_adam {
@@ -236,6 +237,26 @@ int ref_model_step(ref_model *r, double lr, double grad_scale)
 {
 	lm_adam_step_scaled(r->opt, lr, grad_scale);
 	return r->opt->t;
+}
+
+/* lm_save_checkpoint / lm_load_checkpoint (lang/lm_serialize.c:300-331,526-587) on this model. */
+int ref_model_save_checkpoint(ref_model *r, int epoch, int step, const char *path)
+{
+	return lm_save_checkpoint(r->model, r->opt, epoch, step, path);
+}
+
+ref_model *ref_model_load_checkpoint(const char *path, int *epoch, int *step)
+{
+	ref_model *r = calloc(1, sizeof(*r));
+
+	if (!r)
+		return NULL;
+	r->model = lm_load_checkpoint(path, &r->opt, epoch, step);
+	if (!r->model) {
+		free(r);
+		return NULL;
+	}
+	return r;
 }
 
 void ref_model_free(ref_model *r)
