@@ -893,4 +893,18 @@ void anni_gpu_set_stream(void *hip_stream)
 		set_compute_stream((hipStream_t)hip_stream);
 }
 
+int anni_gpu_device_info(char *name, size_t cap, int *driver_version)
+{
+	hipDeviceProp_t prop;
+	int dev = 0;
+
+	if (!device_ready() || !name || cap == 0 || hipGetDevice(&dev) != hipSuccess
+	    || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+		return -1;
+	snprintf(name, cap, "%s (%s)", prop.name[0] ? prop.name : "AMD GPU", prop.gcnArchName);
+	if (driver_version && hipDriverGetVersion(driver_version) != hipSuccess)
+		*driver_version = 0;
+	return 0;
+}
+
 } /* extern "C" */

@@ -96,6 +96,7 @@ _PROTOS = {
     "anni_adam_write_state": (C.c_int, [C.POINTER(Adam), C.c_int, C.c_int, C.c_int]),
     "anni_adam_read_state": (C.c_int, [C.POINTER(Adam), C.c_int, C.POINTER(C.c_int),
                                        C.POINTER(C.c_int)]),
+    "anni_gpu_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int)]),
     "anni_lr_set_schedule": (None, [C.c_int, C.c_int, C.c_char_p]),
     "anni_lr_set_sched_from": (None, [C.c_int]),
     "anni_lr_step": (C.c_double, [C.c_double, C.c_int]),

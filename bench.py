@@ -223,6 +223,9 @@ def main():
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="only run the plain copy kernel over BYTES ten times (counter calibration)")
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds for the CPU legs")
+    ap.add_argument("--ref-jsonl", default=None, metavar="FILE",
+                    help="also append one row in the reference's bench-log schema (optimizer "
+                         "phase only); steps are then timed one call each")
     a = ap.parse_args()
     if a.steps is None:
         a.steps = 10 if a.workload == "555m" else 8
@@ -235,6 +238,10 @@ def main():
     from anni_amd import layout, lib
     from anni_amd.lm_adam import LmAdam
     L = lib.require_gpu()
+    env = None
+    if a.ref_jsonl:
+        from anni_amd import bench_row
+        env = bench_row.probe_env(L, os.path.dirname(os.path.abspath(__file__)))
     if a.copy_calibration:
         copy_calibration(L, a.copy_calibration)
         return
@@ -256,16 +263,20 @@ def main():
     unit = 1.0 / (math.sqrt(n) * 1e-3)
     gss = [unit * (1.7 if s % 2 else 0.6) for s in range(total)]
 
+    per_step_ms, skipped_steps = [], []
+
     def run(first, count, per_kernel):
         ptrs = (C.c_void_p * count)(*[ring[first + i] for i in range(count)])
         lr = (C.c_double * count)(*lrs[first:first + count])
         gs = (C.c_double * count)(*gss[first:first + count])
         ms, ms_a, ms_b = C.c_float(0), C.c_float(0), C.c_float(0)
-        if gt == 2:
+        if gt == 2 or (a.ref_jsonl and per_kernel):
             # fp8: each flat carries its own per-tensor scales -> one call per step
+            # (also when the per-step distribution is wanted)
             tot = sa = sb = 0.0
             for i in range(count):
-                opt.o.d_gscale = scales[first + i].ptr
+                if gt == 2:
+                    opt.o.d_gscale = scales[first + i].ptr
                 one = (C.c_void_p * 1)(ptrs[i])
                 rc = L.anni_adam_time_steps(opt.h, 1, one, 1, C.byref(C.c_double(lr[i])),
                                             C.byref(C.c_double(gs[i])), C.byref(ms),
@@ -273,6 +284,11 @@ def main():
                                             C.byref(ms_b) if per_kernel else None)
                 assert rc == 0, L.gpu_debug_last_error()
                 tot, sa, sb = tot + ms.value, sa + ms_a.value, sb + ms_b.value
+                if per_kernel:
+                    per_step_ms.append(ms.value)
+                    o = opt.sync_stats() if a.ref_jsonl else None
+                    if o is not None and (o.last_skipped or not math.isfinite(o.last_grad_norm)):
+                        skipped_steps.append(first + i)
             return tot, sa, sb
         rc = L.anni_adam_time_steps(opt.h, count, ptrs, count, lr, gs, C.byref(ms),
                                     C.byref(ms_a) if per_kernel else None,
@@ -288,6 +304,10 @@ def main():
     L.gpu_device_sync()
     wall_ms = (time.perf_counter() - t0) * 1e3
 
+    peak_mb = 0.0
+    fr, tt = C.c_size_t(0), C.c_size_t(0)
+    if L.gpu_mem_info(C.byref(fr), C.byref(tt)) == 0:
+        peak_mb = (tt.value - fr.value) / 1048576.0
     st = opt.sync_stats()
     assert opt.t == total and math.isfinite(st.last_grad_norm)
     bpp = norm_bpp + upd_bpp
@@ -336,6 +356,12 @@ def main():
                 out["reference_caller_185m"] = ref_leg
         except Exception as e:                      # the checker must never sink the bench line
             out["reference_caller_185m"] = {"error": repr(e)}
+    if a.ref_jsonl:
+        row = bench_row.adam_row(env, a.workload, size, gt, mt, n, a.warmup, per_step_ms, 3e-4,
+                                 peak_mb, not skipped_steps)
+        bench_row.append(a.ref_jsonl, row)
+        out["ref_jsonl_row"] = row
+        out["vram_used_before_mb"] = env["vram_used_mb"]
     print(json.dumps(out))
     if opt is not None:
         opt.free()

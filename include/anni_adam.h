@@ -155,6 +155,9 @@ double	anni_lr_step(double base_lr, int step);
 void	*anni_gpu_stream(void);
 void	anni_gpu_set_stream(void *hip_stream);
 
+/* Name and architecture of the current device and the HIP driver version: what the reference's bench row records from nvidia-smi (lang/lm_bench.c:287-316). */
+int	anni_gpu_device_info(char *name, size_t cap, int *driver_version);
+
 /*
 ** Times `count` back-to-back steps with HIP events recorded on the compute
 ** stream: per step, the gradient flat grads[i % n_grads] is bound (NULL array =

@@ -148,8 +148,8 @@ def test_block_layout_and_resume(gpu, oracle, tmp_path):
 
 def test_block_equals_reference_checkpoint_and_reference_loads_ours(gpu, oracle, tmp_path):
     """The reference's real model (its compile-time sizes; the byte vocabulary of lm_create, which
-    is what its loader expects of a file without a tokenizer) trained two steps on this backend and saved by its own lm_save_checkpoint: the arena, given the same m / v / t,
-    writes the same optimizer block byte for byte.  Then the other direction: the reference's
+    is what its loader expects of a file without a tokenizer) trained two steps on this backend
+    and saved by its own lm_save_checkpoint: the arena, given the same m / v / t, writes the same optimizer block byte for byte.  Then the other direction: the reference's
     weights section followed by a block written from a different arena state is a file the
     reference's lm_load_checkpoint accepts, and the m / v / t / epoch / step it loads are ours."""
     if not oracle.ref_hip_available():
