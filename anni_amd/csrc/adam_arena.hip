@@ -34,6 +34,14 @@ struct anni_adam_priv {
 	double			probe_gbps;	/* update throughput measured at creation (0: not measured) */
 	std::vector<int64_t>	offsets;
 	std::vector<uint32_t>	flags;
+	/* derived outputs (anni_adam_enable_derived): one more allocation */
+	std::vector<Seg>	segs;		/* host copy of the device table */
+	void			*derived;
+	uint32_t		*d_wamax[2];	/* this step's and the next step's max |p| words */
+	PackDesc		*d_packs;
+	int			der_cur;	/* which of d_wamax the next producer raises */
+	int			fp8_twins;	/* 1: some tensor keeps an E4M3 twin */
+	float			der_ms;		/* E4M3 pass time summed by anni_adam_time_steps */
 };
 
 static size_t elem_bytes(int type)
@@ -317,13 +325,15 @@ anni_adam *anni_adam_create(const anni_tensor *tensors, int n_tensors,
 		for (int i = 0; i < n_tensors; i++) {
 			segs[(size_t)i].begin = at;
 			segs[(size_t)i].end = at + tensors[i].n;
-			segs[(size_t)i].flags = tensors[i].flags;
+			segs[(size_t)i].flags = tensors[i].flags
+			    & (ANNI_T_DECAY | ANNI_T_TWIN | ANNI_T_FP8TWIN);
 			segs[(size_t)i].pad = 0;
 			pv->offsets[(size_t)i] = at;
 			pv->flags[(size_t)i] = tensors[i].flags;
 			at += tensors[i].n;
 		}
 	}
+	pv->segs = segs;
 	/* Launch table: the tensor that holds the first element of each tile. */
 	z.n = n;
 	z.n_tensors = n_tensors;
@@ -422,6 +432,8 @@ void anni_adam_free(anni_adam **popt)
 			(void)hipStreamSynchronize(compute_stream());
 		if (opt->priv->arena)
 			(void)hip_ok(hipFree(opt->priv->arena), "arena hipFree");
+		if (opt->priv->derived)
+			(void)hip_ok(hipFree(opt->priv->derived), "derived hipFree");
 		if (opt->priv->h_state)
 			(void)hip_ok(hipHostFree(opt->priv->h_state), "arena hipHostFree");
 		delete opt->priv;
@@ -462,12 +474,123 @@ double anni_adam_probe_gbps(const anni_adam *opt)
 	return opt && opt->priv ? opt->priv->probe_gbps : 0.0;
 }
 
+static void describe(const anni_adam *opt, Flat *f);
+
+/* The derived outputs as the update would leave them, straight from p. */
+static int derive_now(anni_adam *opt)
+{
+	anni_adam_priv *pv = opt->priv;
+	hipStream_t st = compute_stream();
+	Flat f;
+
+	describe(opt, &f);
+	if (launch_derive(st, f) != 0)
+		return -1;
+	if (pv->fp8_twins) {
+		if (launch_fp8_twins(st, f, (uint8_t *)opt->d_param_fp8, opt->d_wscale,
+		    pv->d_wamax[pv->der_cur], pv->d_wamax[pv->der_cur ^ 1], opt->n_tensors,
+		    nullptr) != 0)
+			return -1;
+		pv->der_cur ^= 1;
+	}
+	return 0;
+}
+
 int anni_adam_seed_twins(anni_adam *opt)
 {
-	if (!opt || !opt->d_param_bf16)
+	if (!opt || !opt->priv || (!opt->d_param_bf16 && !opt->priv->derived))
 		return -1;
-	return launch_f32_to_bf16(compute_stream(), (uint16_t *)opt->d_param_bf16, opt->d_param,
-	    opt->n);
+	if (opt->d_param_bf16 && launch_f32_to_bf16(compute_stream(),
+	    (uint16_t *)opt->d_param_bf16, opt->d_param, opt->n) != 0)
+		return -1;
+	return opt->priv->derived ? derive_now(opt) : 0;
+}
+
+int anni_adam_enable_derived(anni_adam *opt, const anni_pack *packs, int n_packs,
+	int64_t pack_elems)
+{
+	anni_adam_priv *pv;
+	hipStream_t st;
+	std::vector<PackDesc> descs;
+	std::vector<Seg> segs;
+	std::vector<float> ones;
+	size_t off_q, off_scale, off_amax, off_packs, off_pack, total;
+	char *base;
+	bool fp8 = false;
+
+	if (!opt || !opt->priv || opt->priv->derived || n_packs < 0 || (n_packs > 0 && !packs)
+	    || pack_elems < 0 || (n_packs > 0 && pack_elems <= 0) || !device_ready())
+		return -1;
+	pv = opt->priv;
+	segs = pv->segs;
+	descs.assign((size_t)opt->n_tensors, PackDesc{0, 1u, 0u});
+	for (int i = 0; i < opt->n_tensors; i++)
+		if (segs[(size_t)i].flags & kSegFp8Twin)
+			fp8 = true;
+	for (int k = 0; k < n_packs; k++) {
+		const anni_pack &pk = packs[k];
+		int64_t cnt, rows;
+
+		if (pk.tensor < 0 || pk.tensor >= opt->n_tensors || pk.cols <= 0
+		    || pk.dst_stride < pk.cols || pk.dst_offset < 0)
+			return -1;
+		if (segs[(size_t)pk.tensor].flags & kSegPack)
+			return -1;		/* one target per tensor */
+		cnt = segs[(size_t)pk.tensor].end - segs[(size_t)pk.tensor].begin;
+		if (cnt <= 0 || cnt >= ((int64_t)1 << 32) || cnt % pk.cols != 0)
+			return -1;
+		rows = cnt / pk.cols;
+		if (pk.dst_offset + (rows - 1) * (int64_t)pk.dst_stride + pk.cols > pack_elems)
+			return -1;
+		descs[(size_t)pk.tensor].dst_off = pk.dst_offset;
+		descs[(size_t)pk.tensor].cols = (uint32_t)pk.cols;
+		descs[(size_t)pk.tensor].dst_stride = (uint32_t)pk.dst_stride;
+		segs[(size_t)pk.tensor].flags |= kSegPack;
+	}
+	if (!fp8 && n_packs == 0)
+		return -1;		/* nothing to derive */
+	off_q = 0;
+	off_scale = round_up(fp8 ? (size_t)opt->n : 0, 256);
+	off_amax = off_scale + round_up((size_t)opt->n_tensors * sizeof(float), 256);
+	off_packs = off_amax + 2 * round_up((size_t)opt->n_tensors * sizeof(uint32_t), 256);
+	off_pack = round_up(off_packs + (size_t)opt->n_tensors * sizeof(PackDesc), (size_t)2 << 20);
+	total = off_pack + round_up((size_t)pack_elems * 2, 256) + 256;
+	if (hipMalloc(&pv->derived, total) != hipSuccess) {
+		(void)hipGetLastError();
+		pv->derived = nullptr;
+		return -1;
+	}
+	base = (char *)pv->derived;
+	st = compute_stream();
+	ones.assign((size_t)opt->n_tensors, 1.0f);
+	pv->d_wamax[0] = (uint32_t *)(base + off_amax);
+	pv->d_wamax[1] = (uint32_t *)(base + off_amax
+	    + round_up((size_t)opt->n_tensors * sizeof(uint32_t), 256));
+	pv->d_packs = (PackDesc *)(base + off_packs);
+	pv->der_cur = 0;
+	pv->fp8_twins = fp8 ? 1 : 0;
+	if (launch_fill_bytes(st, base, 0, total) != 0
+	    || !hip_ok(hipMemcpyAsync(base + off_scale, ones.data(),
+	    (size_t)opt->n_tensors * sizeof(float), hipMemcpyHostToDevice, st), "wscale")
+	    || !hip_ok(hipMemcpyAsync(pv->d_packs, descs.data(),
+	    (size_t)opt->n_tensors * sizeof(PackDesc), hipMemcpyHostToDevice, st), "packs")
+	    || !hip_ok(hipMemcpyAsync(pv->d_segs, segs.data(), (size_t)opt->n_tensors * sizeof(Seg),
+	    hipMemcpyHostToDevice, st), "segs")
+	    || !hip_ok(hipStreamSynchronize(st), "derived init")) {
+		(void)hipFree(pv->derived);
+		pv->derived = nullptr;
+		return -1;
+	}
+	pv->segs = segs;
+	opt->d_param_fp8 = fp8 ? base + off_q : nullptr;
+	opt->d_wscale = (float *)(base + off_scale);
+	opt->d_pack_bf16 = n_packs ? base + off_pack : nullptr;
+	return 0;
+}
+
+float anni_adam_timed_derived_ms(const anni_adam *opt)
+{
+	return opt && opt->priv ? opt->priv->der_ms : 0.0f;
 }
 
 int anni_adam_zero_grad(anni_adam *opt)
@@ -497,9 +620,14 @@ static void describe(const anni_adam *opt, Flat *f)
 	f->segs = pv->d_segs;
 	f->tile_seg = pv->d_tile_seg;
 	f->gscale = opt->d_gscale;
+	if (pv->derived) {
+		f->der.wamax = pv->fp8_twins ? pv->d_wamax[pv->der_cur] : nullptr;
+		f->der.packs = pv->d_packs;
+		f->der.pack = (uint16_t *)opt->d_pack_bf16;
+	}
 }
 
-/* One step; ev (may be NULL) = three events recorded before, between and after the two launches. */
+/* One step; ev (may be NULL) = four events recorded before, between and after the launches. */
 static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *ev)
 {
 	anni_adam_priv *pv;
@@ -552,6 +680,15 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 		return -1;
 	if (ev)
 		(void)hipEventRecord(ev[2], st);
+	if (pv->fp8_twins) {
+		if (launch_fp8_twins(st, f, (uint8_t *)opt->d_param_fp8, opt->d_wscale,
+		    pv->d_wamax[pv->der_cur], pv->d_wamax[pv->der_cur ^ 1], opt->n_tensors,
+		    norm.use_norm ? pv->d_state : nullptr) != 0)
+			return -1;
+		pv->der_cur ^= 1;
+	}
+	if (ev)
+		(void)hipEventRecord(ev[3], st);
 	return 0;
 }
 
@@ -602,7 +739,7 @@ int anni_adam_time_steps(anni_adam *opt, int count, void *const *grads, int n_gr
 	if (grads && n_grads <= 0)
 		return -1;
 	st = compute_stream();
-	ev.resize(per_kernel ? (size_t)count * 3 : 2);
+	ev.resize(per_kernel ? (size_t)count * 4 : 2);
 	for (size_t i = 0; i < ev.size(); i++)
 		if (hipEventCreate(&ev[i]) != hipSuccess) {
 			for (size_t k = 0; k < i; k++)
@@ -614,7 +751,7 @@ int anni_adam_time_steps(anni_adam *opt, int count, void *const *grads, int n_gr
 	for (int i = 0; i < count && rc == 0; i++) {
 		if (grads)
 			(void)anni_adam_bind_grad(opt, grads[i % n_grads]);
-		rc = step_impl(opt, lr[i], grad_scale[i], per_kernel ? &ev[(size_t)i * 3] : nullptr);
+		rc = step_impl(opt, lr[i], grad_scale[i], per_kernel ? &ev[(size_t)i * 4] : nullptr);
 		if (rc == 1)
 			rc = -1;		/* a timed run must not contain no-op steps */
 	}
@@ -626,17 +763,20 @@ int anni_adam_time_steps(anni_adam *opt, int count, void *const *grads, int n_gr
 		float ms = 0.0f;
 
 		if (per_kernel) {
-			float a = 0.0f, b = 0.0f;
+			float a = 0.0f, b = 0.0f, d = 0.0f;
 
 			for (int i = 0; i < count; i++) {
-				float x = 0.0f, y = 0.0f;
+				float x = 0.0f, y = 0.0f, w = 0.0f;
 
-				(void)hipEventElapsedTime(&x, ev[(size_t)i * 3], ev[(size_t)i * 3 + 1]);
-				(void)hipEventElapsedTime(&y, ev[(size_t)i * 3 + 1], ev[(size_t)i * 3 + 2]);
+				(void)hipEventElapsedTime(&x, ev[(size_t)i * 4], ev[(size_t)i * 4 + 1]);
+				(void)hipEventElapsedTime(&y, ev[(size_t)i * 4 + 1], ev[(size_t)i * 4 + 2]);
+				(void)hipEventElapsedTime(&w, ev[(size_t)i * 4 + 2], ev[(size_t)i * 4 + 3]);
 				a += x;
 				b += y;
+				d += w;
 			}
-			(void)hipEventElapsedTime(&ms, ev[0], ev[(size_t)count * 3 - 1]);
+			opt->priv->der_ms = d;
+			(void)hipEventElapsedTime(&ms, ev[0], ev[(size_t)count * 4 - 1]);
 			if (ms_sumsq)
 				*ms_sumsq = a;
 			if (ms_update)

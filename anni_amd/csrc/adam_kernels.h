@@ -32,6 +32,8 @@ constexpr int kMaxPartials = 8192;		/* upper bound on the sum-of-squares grid */
 
 constexpr uint32_t kSegDecay = 1u;		/* decoupled weight decay applies */
 constexpr uint32_t kSegTwin = 2u;		/* bf16 twin is written */
+constexpr uint32_t kSegFp8Twin = 4u;		/* E4M3 twin with a per-tensor scale is kept current */
+constexpr uint32_t kSegPack = 8u;		/* bf16 of the tensor also goes into a packed matrix */
 
 /* One tensor of the flat: elements [begin, end). */
 struct Seg {
@@ -39,6 +41,26 @@ struct Seg {
 	int64_t		end;
 	uint32_t	flags;
 	uint32_t	pad;
+};
+
+/*
+** Where the bf16 of a row-major matrix of `cols` columns also goes: element (r, c) lands at
+** pack[dst_off + r * dst_stride + c] (the [Wq | Wk | Wv] operand of num/gpu_cuda.cu:6456-6470).
+*/
+struct PackDesc {
+	int64_t		dst_off;
+	uint32_t	cols;
+	uint32_t	dst_stride;
+};
+
+/*
+** Outputs derived from the new weights in the same pass (all NULL: none).  wamax[s] receives
+** max |p| of tensor s as unsigned bits through atomic max (order independent, so deterministic).
+*/
+struct Derived {
+	uint32_t	*wamax;
+	const PackDesc	*packs;		/* one per tensor, read for tensors flagged kSegPack */
+	uint16_t	*pack;
 };
 
 /* Written by the step on the device; read back only when the host asks. */
@@ -64,6 +86,7 @@ struct Flat {
 	const int32_t	*tile_seg;	/* NULL when segs is NULL */
 	const float	*gscale;	/* per-tensor dequant scale (fp8 gradients) */
 	uint32_t	uniform_flags;
+	Derived		der;
 };
 
 /* How the update obtains the global norm (use_norm == 0: grad_scale is final). */
@@ -87,6 +110,18 @@ int	launch_finalize(hipStream_t st, const double *partials, int n_partials, doub
 		int skip_nonfinite, double grad_scale, StepState *state);
 int	launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double grad_scale,
 		const NormIn &norm);
+/*
+** Derived outputs straight from p, without an update (after weights were loaded):
+** wamax and the packed matrices as the update would leave them.
+*/
+int	launch_derive(hipStream_t st, const Flat &f);
+/*
+** q = E4M3(p * (1 / scale_s)) for the tensors flagged kSegFp8Twin, scale_s from wamax[s]
+** (num/gpu_cuda.cu:826-851,927-938); wscale[s] receives the scale, wamax_next[0..n_tensors) is
+** cleared for the following step.  state (may be NULL): a skipped step leaves q and wscale alone.
+*/
+int	launch_fp8_twins(hipStream_t st, const Flat &f, uint8_t *q, float *wscale,
+		const uint32_t *wamax, uint32_t *wamax_next, int n_tensors, const StepState *state);
 int	launch_f32_to_bf16(hipStream_t st, uint16_t *dst, const float *src, int64_t n);
 /* pairs[2k] = m[first+k], pairs[2k+1] = v[first+k] as floats (bf16 moments widen exactly). */
 int	launch_mv_interleave(hipStream_t st, float *pairs, const void *m, const void *v,

@@ -160,6 +160,62 @@ __device__ __forceinline__ double partials_sum(const double *partials, int np, d
 	return block_sum(acc, lds);
 }
 
+/* ---- derived outputs ------------------------------------------------------ */
+
+/* Max over the 64 lanes of a wavefront; lane 0 holds it. */
+__device__ __forceinline__ float wave_max(float x)
+{
+#pragma unroll
+	for (int off = 32; off > 0; off >>= 1)
+		x = fmaxf(x, __shfl_down(x, off, 64));
+	return x;
+}
+
+/* max |x| of four values; NaNs are ignored (fmaxf returns the other operand). */
+__device__ __forceinline__ float amax4(float acc, f32x4 x)
+{
+	return fmaxf(acc, fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w))));
+}
+
+/*
+** Raises *word to the bits of m (m > 0, not NaN; such floats order like unsigned integers).
+** The word only grows during a launch, so a stale read costs at most a redundant atomic.
+*/
+__device__ __forceinline__ void amax_raise(uint32_t *word, float m)
+{
+	const uint32_t bits = __float_as_uint(m);
+
+	if (bits > __atomic_load_n(word, __ATOMIC_RELAXED))
+		atomicMax(word, bits);
+}
+
+/* bf16 of element e of a packed tensor into its place in the packed matrix. */
+__device__ __forceinline__ void pack_one(uint16_t *pack, const PackDesc &pd, uint32_t e, float x)
+{
+	const uint32_t r = e / pd.cols;
+	const uint32_t c = e - r * pd.cols;
+
+	pack[pd.dst_off + (int64_t)r * pd.dst_stride + c] = (uint16_t)bf16_rne(x);
+}
+
+/* The same for elements e..e+3: one 8-byte store when they share a row and the target is aligned. */
+template <bool NT>
+__device__ __forceinline__ void pack_quad(uint16_t *pack, const PackDesc &pd, uint32_t e, f32x4 x)
+{
+	const uint32_t r = e / pd.cols;
+	const uint32_t c = e - r * pd.cols;
+	const int64_t d = pd.dst_off + (int64_t)r * pd.dst_stride + c;
+
+	if (c + kQuad <= pd.cols && (d & 3) == 0) {
+		store_quad<kBF16, NT>(pack, d, x);
+	} else {
+		pack_one(pack, pd, e, x.x);
+		pack_one(pack, pd, e + 1, x.y);
+		pack_one(pack, pd, e + 2, x.z);
+		pack_one(pack, pd, e + 3, x.w);
+	}
+}
+
 struct NormOut {
 	double	gs;
 	bool	skip;
@@ -382,6 +438,7 @@ struct UpdateArgs {
 	int		n_partials;
 	double		clip;
 	StepState	*state;
+	Derived		der;
 };
 
 /*
@@ -389,7 +446,7 @@ struct UpdateArgs {
 ** types the kernel moves fewer bytes per element for the same arithmetic, so those modes
 ** take the cheaper constant division (adam_math.h) and the deeper unroll.
 */
-template <int GT, int MT, int U, bool NT>
+template <int GT, int MT, int U, bool NT, bool DER>
 __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 {
 	__shared__ double lds[4];
@@ -434,7 +491,16 @@ __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 			const bool decay = a.c.decay_on && (flags & kSegDecay) != 0;
 			const bool twin = (flags & kSegTwin) != 0 && a.twin != nullptr;
 			const float sc = (GT == kFP8) ? a.gscale[s] : 1.0f;
+			const bool fp8w = DER && (flags & kSegFp8Twin) != 0 && a.der.wamax != nullptr;
+			const bool pk = DER && (flags & kSegPack) != 0 && a.der.pack != nullptr;
+			PackDesc pd = {0, 1u, 0u};
+			int64_t seg_begin = 0;
+			float amax_l = 0.0f;
 
+			if (pk) {
+				pd = a.der.packs[s];
+				seg_begin = a.segs[s].begin;
+			}
 #pragma unroll
 			for (int sub = 0; sub < kQuadsPerTile / U; sub++) {
 				f32x4 P[U], G[U], M[U], V[U];
@@ -468,7 +534,16 @@ __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 					zero_quad<GT, NT>(a.g, idx[u]);
 					if (twin)
 						store_quad<kBF16, NT>(a.twin, idx[u], P[u]);
+					if (fp8w)
+						amax_l = amax4(amax_l, P[u]);
+					if (pk)
+						pack_quad<NT>(a.der.pack, pd, (uint32_t)(idx[u] - seg_begin), P[u]);
 				}
+			}
+			if (fp8w) {
+				amax_l = wave_max(amax_l);
+				if ((tid & 63) == 0 && amax_l > 0.0f)
+					amax_raise(a.der.wamax + s, amax_l);
 			}
 		} else {
 			for (int64_t i = base + tid; i < end; i += kThreads) {
@@ -492,6 +567,155 @@ __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 				zero_one<GT>(a.g, i);
 				if ((flags & kSegTwin) != 0 && a.twin != nullptr)
 					a.twin[i] = (uint16_t)bf16_rne(e.p);
+				if (DER && (flags & kSegFp8Twin) != 0 && a.der.wamax != nullptr) {
+					const float ab = fmaxf(0.0f, fabsf(e.p));
+
+					if (ab > 0.0f)
+						amax_raise(a.der.wamax + s, ab);
+				}
+				if (DER && (flags & kSegPack) != 0 && a.der.pack != nullptr)
+					pack_one(a.der.pack, a.der.packs[s], (uint32_t)(i - a.segs[s].begin), e.p);
+			}
+		}
+	}
+}
+
+/* ---- derived outputs without an update, and the E4M3 twins ----------------------- */
+
+struct DeriveArgs {
+	const float	*p;
+	int64_t		n;
+	const Seg	*segs;
+	const int32_t	*tile_seg;
+	Derived		der;
+	int		vec_ok;
+};
+
+template <bool NT>
+__global__ __launch_bounds__(kThreads) void derive_kernel(DeriveArgs a)
+{
+	const int tid = threadIdx.x;
+	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
+
+	for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+		const int64_t base = tile * kTile;
+		const int64_t end = base + kTile < a.n ? base + kTile : a.n;
+		int s = a.tile_seg[tile];
+
+		if (a.vec_ok && end - base == kTile && a.segs[s].end >= end) {
+			const uint32_t flags = a.segs[s].flags;
+			const bool fp8w = (flags & kSegFp8Twin) != 0 && a.der.wamax != nullptr;
+			const bool pk = (flags & kSegPack) != 0 && a.der.pack != nullptr;
+			float amax_l = 0.0f;
+
+			if (!fp8w && !pk)
+				continue;
+			const PackDesc pd = pk ? a.der.packs[s] : PackDesc{0, 1u, 0u};
+			const int64_t seg_begin = a.segs[s].begin;
+
+#pragma unroll
+			for (int u = 0; u < kQuadsPerTile; u++) {
+				const int64_t idx = base + (int64_t)(u * kThreads + tid) * kQuad;
+				const f32x4 P = load_quad<kF32, NT>(a.p, idx, 1.0f);
+
+				if (fp8w)
+					amax_l = amax4(amax_l, P);
+				if (pk)
+					pack_quad<NT>(a.der.pack, pd, (uint32_t)(idx - seg_begin), P);
+			}
+			if (fp8w) {
+				amax_l = wave_max(amax_l);
+				if ((tid & 63) == 0 && amax_l > 0.0f)
+					amax_raise(a.der.wamax + s, amax_l);
+			}
+		} else {
+			for (int64_t i = base + tid; i < end; i += kThreads) {
+				while (i >= a.segs[s].end)
+					s++;
+				const uint32_t flags = a.segs[s].flags;
+				const float x = a.p[i];
+
+				if ((flags & kSegFp8Twin) != 0 && a.der.wamax != nullptr) {
+					const float ab = fmaxf(0.0f, fabsf(x));
+
+					if (ab > 0.0f)
+						amax_raise(a.der.wamax + s, ab);
+				}
+				if ((flags & kSegPack) != 0 && a.der.pack != nullptr)
+					pack_one(a.der.pack, a.der.packs[s], (uint32_t)(i - a.segs[s].begin), x);
+			}
+		}
+	}
+}
+
+struct Fp8TwinArgs {
+	const float	*p;
+	uint8_t		*q;
+	int64_t		n;
+	const Seg	*segs;
+	const int32_t	*tile_seg;
+	const uint32_t	*wamax;
+	uint32_t	*wamax_next;
+	float		*wscale;
+	int		n_tensors;
+	const StepState	*state;
+	int		vec_ok;
+};
+
+/*
+** The quantisation pass of the E4M3 twins.  The scale of a tensor needs the max over ALL of
+** its new values, which the update has just reduced into wamax, so this pass reads p once
+** more (4 bytes) and writes 1 byte per element, where amax + quantise as separate passes
+** over p would read it twice.
+*/
+template <bool NT>
+__global__ __launch_bounds__(kThreads) void fp8_twin_kernel(Fp8TwinArgs a)
+{
+	const int tid = threadIdx.x;
+	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
+	const bool skipped = a.state != nullptr && a.state->skipped != 0;
+
+	if (blockIdx.x == 0) {
+		for (int s = tid; s < a.n_tensors; s += kThreads) {
+			if (!skipped && (a.segs[s].flags & kSegFp8Twin) != 0)
+				a.wscale[s] = scale_from_amax(__uint_as_float(a.wamax[s]));
+			a.wamax_next[s] = 0u;
+		}
+	}
+	if (skipped)
+		return;		/* p did not change: the twins and their scales stay */
+	for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+		const int64_t base = tile * kTile;
+		const int64_t end = base + kTile < a.n ? base + kTile : a.n;
+		int s = a.tile_seg[tile];
+
+		if (a.vec_ok && end - base == kTile && a.segs[s].end >= end) {
+			if ((a.segs[s].flags & kSegFp8Twin) == 0)
+				continue;
+			const float inv = 1.0f / scale_from_amax(__uint_as_float(a.wamax[s]));
+			f32x4 P[kQuadsPerTile];
+
+#pragma unroll
+			for (int u = 0; u < kQuadsPerTile; u++)
+				P[u] = load_quad<kF32, NT>(a.p, base + (int64_t)(u * kThreads + tid) * kQuad, 1.0f);
+#pragma unroll
+			for (int u = 0; u < kQuadsPerTile; u++) {
+				const uint32_t w = fp8_e4m3_encode(P[u].x * inv)
+				    | (fp8_e4m3_encode(P[u].y * inv) << 8)
+				    | (fp8_e4m3_encode(P[u].z * inv) << 16)
+				    | (fp8_e4m3_encode(P[u].w * inv) << 24);
+
+				st<NT>((uint32_t *)(a.q + base + (int64_t)(u * kThreads + tid) * kQuad), w);
+			}
+		} else {
+			for (int64_t i = base + tid; i < end; i += kThreads) {
+				while (i >= a.segs[s].end)
+					s++;
+				if ((a.segs[s].flags & kSegFp8Twin) != 0) {
+					const float inv = 1.0f / scale_from_amax(__uint_as_float(a.wamax[s]));
+
+					a.q[i] = (uint8_t)fp8_e4m3_encode(a.p[i] * inv);
+				}
 			}
 		}
 	}
@@ -730,12 +954,34 @@ static void update_launch(hipStream_t st, int grid, const UpdateArgs &a)
 {
 	constexpr int U = (GT == kF32 && MT == kF32) ? ANNI_UPDATE_UNROLL : ANNI_UPDATE_UNROLL_NARROW;
 
-	if (nt_on())
-		hipLaunchKernelGGL((adam_update_kernel<GT, MT, U, true>), dim3(grid), dim3(kThreads),
-		    0, st, a);
-	else
-		hipLaunchKernelGGL((adam_update_kernel<GT, MT, U, false>), dim3(grid), dim3(kThreads),
-		    0, st, a);
+	const bool der = a.der.wamax != nullptr || a.der.pack != nullptr;
+
+	if (der) {
+		if (nt_on())
+			hipLaunchKernelGGL((adam_update_kernel<GT, MT, U, true, true>), dim3(grid),
+			    dim3(kThreads), 0, st, a);
+		else
+			hipLaunchKernelGGL((adam_update_kernel<GT, MT, U, false, true>), dim3(grid),
+			    dim3(kThreads), 0, st, a);
+	} else if (nt_on()) {
+		hipLaunchKernelGGL((adam_update_kernel<GT, MT, U, true, false>), dim3(grid),
+		    dim3(kThreads), 0, st, a);
+	} else {
+		hipLaunchKernelGGL((adam_update_kernel<GT, MT, U, false, false>), dim3(grid),
+		    dim3(kThreads), 0, st, a);
+	}
+}
+
+/* Derived outputs need the launch table, an 8-byte aligned pack flat and descriptors for it. */
+static int check_derived(const Flat &f)
+{
+	if (!f.der.wamax && !f.der.pack)
+		return 0;
+	if (!f.segs || !f.tile_seg)
+		return -1;
+	if (f.der.pack && (!f.der.packs || !aligned(f.der.pack, 8)))
+		return -1;
+	return 0;
 }
 
 int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double grad_scale,
@@ -744,7 +990,7 @@ int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double gra
 	UpdateArgs a;
 	int grid;
 
-	if (check_flat(f, true) != 0)
+	if (check_flat(f, true) != 0 || check_derived(f) != 0)
 		return -1;
 	if (norm.use_norm && (!norm.partials || norm.n_partials <= 0))
 		return -1;
@@ -770,6 +1016,7 @@ int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double gra
 	a.n_partials = norm.n_partials;
 	a.clip = norm.clip;
 	a.state = norm.state;
+	a.der = f.der;
 	if (f.moment_type == kF32) {
 		if (f.grad_type == kF32)
 			update_launch<kF32, kF32>(st, grid, a);
@@ -806,6 +1053,51 @@ int launch_f32_to_bf16(hipStream_t st, uint16_t *dst, const float *src, int64_t 
 		return -1;
 	hipLaunchKernelGGL(f32_to_bf16_kernel, dim3(helper_grid(n / kQuad + 1)), dim3(kThreads),
 	    0, st, dst, src, n, aligned(src, 16) && aligned(dst, 8) ? 1 : 0);
+	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int launch_derive(hipStream_t st, const Flat &f)
+{
+	DeriveArgs a;
+
+	if (!f.p || f.n <= 0 || check_derived(f) != 0 || (!f.der.wamax && !f.der.pack))
+		return -1;
+	a.p = f.p;
+	a.n = f.n;
+	a.segs = f.segs;
+	a.tile_seg = f.tile_seg;
+	a.der = f.der;
+	a.vec_ok = aligned(f.p, 16) ? 1 : 0;
+	if (nt_on())
+		hipLaunchKernelGGL((derive_kernel<true>), dim3(grid_for(f.n)), dim3(kThreads), 0, st, a);
+	else
+		hipLaunchKernelGGL((derive_kernel<false>), dim3(grid_for(f.n)), dim3(kThreads), 0, st, a);
+	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int launch_fp8_twins(hipStream_t st, const Flat &f, uint8_t *q, float *wscale,
+	const uint32_t *wamax, uint32_t *wamax_next, int n_tensors, const StepState *state)
+{
+	Fp8TwinArgs a;
+
+	if (!f.p || f.n <= 0 || !f.segs || !f.tile_seg || !q || !wscale || !wamax || !wamax_next
+	    || n_tensors <= 0)
+		return -1;
+	a.p = f.p;
+	a.q = q;
+	a.n = f.n;
+	a.segs = f.segs;
+	a.tile_seg = f.tile_seg;
+	a.wamax = wamax;
+	a.wamax_next = wamax_next;
+	a.wscale = wscale;
+	a.n_tensors = n_tensors;
+	a.state = state;
+	a.vec_ok = aligned(f.p, 16) && aligned(q, 4) ? 1 : 0;
+	if (nt_on())
+		hipLaunchKernelGGL((fp8_twin_kernel<true>), dim3(grid_for(f.n)), dim3(kThreads), 0, st, a);
+	else
+		hipLaunchKernelGGL((fp8_twin_kernel<false>), dim3(grid_for(f.n)), dim3(kThreads), 0, st, a);
 	return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

@@ -142,5 +142,19 @@ __device__ __forceinline__ uint32_t fp8_e4m3_encode(float x)
 	return s | (uint32_t)((e + 7) << 3) | (uint32_t)(q - 8);
 }
 
+/*
+** Per-tensor FP8 scale from the tensor's max |x| (num/gpu_cuda.cu:927-938): amax / 448, at
+** least 1e-12; a zero, negative or non-finite amax counts as 1e-8.
+*/
+__device__ __forceinline__ float scale_from_amax(float a)
+{
+	if (!(a > 0.0f) || !(a <= 3.4028234663852886e38f))
+		a = 1e-8f;
+	a = a / 448.0f;
+	if (a < 1e-12f)
+		a = 1e-12f;
+	return a;
+}
+
 } /* namespace anni */
 #endif

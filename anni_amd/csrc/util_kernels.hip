@@ -67,16 +67,6 @@ __global__ __launch_bounds__(kThreads) void amax_kernel(uint32_t *amax, const fl
 	}
 }
 
-__device__ __forceinline__ float scale_from_amax(float a)
-{
-	if (!(a > 0.0f) || !(a <= 3.4028234663852886e38f))
-		a = 1e-8f;
-	a = a / 448.0f;
-	if (a < 1e-12f)
-		a = 1e-12f;
-	return a;
-}
-
 /* In place: the amax word becomes the tensor's scale. */
 __global__ void amax_to_scale_kernel(float *word)
 {

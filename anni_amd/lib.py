@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(HERE, "libanni_gpu_hip.so")
 
 F32, BF16, FP8_E4M3 = 0, 1, 2
-T_DECAY, T_TWIN = 1, 2
+T_DECAY, T_TWIN, T_FP8TWIN = 1, 2, 4
 LAYOUT_AUTO, LAYOUT_COMPACT, LAYOUT_SPREAD = 0, 1, 2
 GPU_PREC_FP32, GPU_PREC_BF16 = 0, 1
 
@@ -40,7 +40,14 @@ class Adam(C.Structure):
                 ("last_clipped", C.c_int), ("cfg", Config),
                 ("d_param", C.c_void_p), ("d_param_bf16", C.c_void_p),
                 ("d_grad", C.c_void_p), ("d_m", C.c_void_p), ("d_v", C.c_void_p),
-                ("d_gscale", C.c_void_p), ("priv", C.c_void_p)]
+                ("d_gscale", C.c_void_p), ("d_param_fp8", C.c_void_p), ("d_wscale", C.c_void_p),
+                ("d_pack_bf16", C.c_void_p), ("priv", C.c_void_p)]
+
+
+class Pack(C.Structure):
+    """anni_pack: a second home for the bf16 of a matrix inside a packed matrix."""
+    _fields_ = [("tensor", C.c_int), ("cols", C.c_int32), ("dst_offset", C.c_int64),
+                ("dst_stride", C.c_int32)]
 
 
 # name -> (restype, argtypes) for every entry point the Python side calls.
@@ -96,6 +103,8 @@ _PROTOS = {
     "anni_adam_write_state": (C.c_int, [C.POINTER(Adam), C.c_int, C.c_int, C.c_int]),
     "anni_adam_read_state": (C.c_int, [C.POINTER(Adam), C.c_int, C.POINTER(C.c_int),
                                        C.POINTER(C.c_int)]),
+    "anni_adam_enable_derived": (C.c_int, [C.POINTER(Adam), C.POINTER(Pack), C.c_int, C.c_int64]),
+    "anni_adam_timed_derived_ms": (C.c_float, [C.POINTER(Adam)]),
     "anni_gpu_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int)]),
     "anni_lr_set_schedule": (None, [C.c_int, C.c_int, C.c_char_p]),
     "anni_lr_set_sched_from": (None, [C.c_int]),

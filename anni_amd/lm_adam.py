@@ -116,6 +116,14 @@ class LmAdam:
         if self.L.anni_adam_seed_twins(self.h) != 0:
             raise RuntimeError("anni_adam_seed_twins failed")
 
+    def enable_derived(self, packs=(), pack_elems=0):
+        """packs: (tensor, cols, dst_offset, dst_stride) tuples; E4M3 twins follow the tensor flags."""
+        arr = (_l.Pack * max(len(packs), 1))(*[_l.Pack(*[int(x) for x in pk]) for pk in packs])
+        if self.L.anni_adam_enable_derived(self.h, arr if packs else None, len(packs),
+                                           int(pack_elems)) != 0:
+            raise RuntimeError("anni_adam_enable_derived refused")
+        self.pack_elems = int(pack_elems)
+
     def sync_stats(self):
         if self.L.anni_adam_sync_stats(self.h) != 0:
             raise RuntimeError("anni_adam_sync_stats failed")
@@ -179,7 +187,9 @@ class LmAdam:
         o = self.o
         return {"param": (o.d_param, np.float32), "grad": (o.d_grad, _NP[self.grad_type]),
                 "m": (o.d_m, _NP[self.moment_type]), "v": (o.d_v, _NP[self.moment_type]),
-                "twin": (o.d_param_bf16, np.uint16), "gscale": (o.d_gscale, np.float32)}[which]
+                "twin": (o.d_param_bf16, np.uint16), "gscale": (o.d_gscale, np.float32),
+                "fp8twin": (o.d_param_fp8, np.uint8), "wscale": (o.d_wscale, np.float32),
+                "pack": (o.d_pack_bf16, np.uint16)}[which]
 
     def upload(self, which, arr, offset=0):
         ptr, dt = self._flat(which)
@@ -191,7 +201,8 @@ class LmAdam:
     def download(self, which, count=None, offset=0):
         ptr, dt = self._flat(which)
         if count is None:
-            count = self.o.n_tensors if which == "gscale" else self.n
+            count = (self.o.n_tensors if which in ("gscale", "wscale")
+                     else self.pack_elems if which == "pack" else self.n)
         out = np.empty(count, dtype=dt)
         if self.L.gpu_memcpy_d2h(out.ctypes.data, ptr + offset * out.itemsize, out.nbytes) != 0:
             raise RuntimeError("download(%s) failed" % which)

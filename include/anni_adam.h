@@ -54,6 +54,7 @@ extern "C" {
 /* Tensor flags. */
 #define ANNI_T_DECAY	1u	/* decoupled weight decay applies (BASELINE: matrices only) */
 #define ANNI_T_TWIN	2u	/* the bf16 twin of this tensor is written */
+#define ANNI_T_FP8TWIN	4u	/* an E4M3 twin with its own scale is kept current (needs anni_adam_enable_derived) */
 
 /* One registered tensor; tensors are packed in registration order with no padding (lm_adam.c:25-57). */
 typedef struct anni_tensor {
@@ -69,6 +70,19 @@ typedef struct anni_adam_config {
 	int	grad_slots;	/* gradient flats the arena allocates (slot 0 starts bound); 0: bind one with anni_adam_bind_grad */
 	int	layout;		/* ANNI_LAYOUT_AUTO / _COMPACT / _SPREAD */
 } anni_adam_config;
+
+/*
+** A second home for the bf16 of a row-major matrix: element (r, c) of tensor `tensor`, which
+** has `cols` columns, also goes to pack[dst_offset + r * dst_stride + c].  Three of these with
+** dst_stride = 3 D and dst_offset = 0, D, 2 D build the [Wq | Wk | Wv] operand that the
+** reference rebuilds from the three twins after each step (num/gpu_cuda.cu:6456-6470,6483-6517).
+*/
+typedef struct anni_pack {
+	int	tensor;
+	int32_t	cols;
+	int64_t	dst_offset;
+	int32_t	dst_stride;
+} anni_pack;
 
 struct anni_adam_priv;
 
@@ -94,6 +108,10 @@ typedef struct anni_adam {
 	void	*d_m;
 	void	*d_v;
 	float	*d_gscale;	/* per-tensor fp8 dequant scale (n_tensors floats) */
+	/* derived outputs, NULL until anni_adam_enable_derived */
+	void	*d_param_fp8;	/* E4M3 twins: n bytes, tensor i at byte anni_adam_tensor_offset(i) */
+	float	*d_wscale;	/* their per-tensor scales (n_tensors floats; 1 for tensors without a twin) */
+	void	*d_pack_bf16;	/* the packed bf16 matrices */
 	struct anni_adam_priv *priv;
 } anni_adam;
 
@@ -116,7 +134,23 @@ int	anni_adam_is_spread(const anni_adam *opt);
 double	anni_adam_probe_gbps(const anni_adam *opt);
 /* Use another gradient flat: a slot of the arena or an external one (n elements of grad_type); NULL = slot 0. */
 int	anni_adam_bind_grad(anni_adam *opt, void *d_grad);
-/* gpu_adam_seed_bf16_flat: twins = bf16(p) for the whole flat (after loading weights). */
+/*
+** Producers of the step's neighbours, fused into the step (no counterpart as code in the
+** reference, which rebuilds both after the step: the E4M3 weight copies by an amax pass and a
+** quantise pass over p per matrix, num/gpu_cuda.cu:1090-1115,1187-1262, the packed QKV operand
+** by a kernel per layer, :6456-6517; docs/low-precision-plan.md:31 asks for this fusion).
+** After this call every step also
+**   - writes bf16(p) of each packed tensor into its place in d_pack_bf16 (pack_elems bf16), and
+**   - keeps q = satfinite_e4m3(p * (1 / scale)), scale = max(amax / 448, 1e-12), current for
+**     the tensors flagged ANNI_T_FP8TWIN: the update reduces max |p| per tensor while it
+**     holds the new values, one more launch reads p and writes q and d_wscale.  The bytes and
+**     scales equal what the reference's fp8_quant_now gives on the new weights.
+** A step skipped for a non-finite norm leaves both as they are.  Call once, before
+** anni_adam_seed_twins; -1 when nothing is flagged and no pack is given, or on a bad descriptor.
+*/
+int	anni_adam_enable_derived(anni_adam *opt, const anni_pack *packs, int n_packs,
+		int64_t pack_elems);
+/* gpu_adam_seed_bf16_flat: twins = bf16(p) for the whole flat (after loading weights); also seeds the derived outputs. */
 int	anni_adam_seed_twins(anni_adam *opt);
 /* lm_adam_zero_grad: clears the gradient flat on the stream. */
 int	anni_adam_zero_grad(anni_adam *opt);
@@ -168,6 +202,8 @@ int	anni_gpu_device_info(char *name, size_t cap, int *driver_version);
 int	anni_adam_time_steps(anni_adam *opt, int count, void *const *grads, int n_grads,
 		const double *lr, const double *grad_scale, float *ms_total,
 		float *ms_sumsq, float *ms_update);
+/* Summed duration of the E4M3 twin launches of the last anni_adam_time_steps run that asked for per-kernel times. */
+float	anni_adam_timed_derived_ms(const anni_adam *opt);
 
 /* ---- producers either side of the step (device utilities) ---------------- */
 
