@@ -34,11 +34,19 @@ struct anni_adam_priv {
 	double			probe_gbps;	/* update throughput measured at creation (0: not measured) */
 	std::vector<int64_t>	offsets;
 	std::vector<uint32_t>	flags;
-	/* derived outputs (anni_adam_enable_derived): one more allocation */
+	char			*hole;		/* spread: unused rest of the tables' region (NULL: none) */
+	size_t			hole_bytes;
+	/*
+	** derived outputs (anni_adam_enable_derived): in the hole of a spread arena, which
+	** keeps them a region away from p, m, v, the twins and the gradients; else one more
+	** allocation
+	*/
 	std::vector<Seg>	segs;		/* host copy of the device table */
 	void			*derived;
+	int			derived_owned;	/* 1: derived is an allocation of its own */
 	uint32_t		*d_wamax[2];	/* this step's and the next step's max |p| words */
 	PackDesc		*d_packs;
+	float			*d_tile_amax;	/* per-wavefront max |p| of every whole tile */
 	int			der_cur;	/* which of d_wamax the next producer raises */
 	int			fp8_twins;	/* 1: some tensor keeps an E4M3 twin */
 	float			der_ms;		/* E4M3 pass time summed by anni_adam_time_steps */
@@ -89,6 +97,7 @@ struct Placement {
 	size_t	off_p, off_m, off_v, off_twin, off_g, off_gscale, off_segs, off_tiles, off_part,
 		off_state;
 	int	spread;
+	size_t	hole_off, hole_bytes;	/* spread: the rest of the tables' region, reserved and unused */
 	double	gbps;		/* what the probe measured (0: not probed) */
 };
 
@@ -156,6 +165,10 @@ static bool place(const Sizes &z, bool spread, Placement *pl)
 	pl->off_part = pl->off_tiles + round_up((size_t)z.n_tiles * sizeof(int32_t), 256);
 	pl->off_state = pl->off_part + round_up((size_t)kMaxPartials * sizeof(double), 256);
 	pl->spread = spread ? 1 : 0;
+	if (spread) {
+		pl->hole_off = round_up(pl->off_state + 256, big);
+		pl->hole_bytes = 4 * stride > pl->hole_off ? 4 * stride - pl->hole_off : 0;
+	}
 	if (hipMalloc(&pl->arena, pl->total) != hipSuccess) {
 		(void)hipGetLastError();
 		pl->arena = nullptr;
@@ -173,6 +186,8 @@ static void adopt(anni_adam *opt, const Sizes &z, const Placement &pl)
 	pv->arena = pl.arena;
 	pv->arena_bytes = pl.total;
 	pv->spread = pl.spread;
+	pv->hole = pl.hole_bytes ? base + pl.hole_off : nullptr;
+	pv->hole_bytes = pl.hole_bytes;
 	pv->probe_gbps = pl.gbps;
 	opt->d_param = (float *)(base + pl.off_p);
 	opt->d_m = base + pl.off_m;
@@ -432,7 +447,7 @@ void anni_adam_free(anni_adam **popt)
 			(void)hipStreamSynchronize(compute_stream());
 		if (opt->priv->arena)
 			(void)hip_ok(hipFree(opt->priv->arena), "arena hipFree");
-		if (opt->priv->derived)
+		if (opt->priv->derived && opt->priv->derived_owned)
 			(void)hip_ok(hipFree(opt->priv->derived), "derived hipFree");
 		if (opt->priv->h_state)
 			(void)hip_ok(hipHostFree(opt->priv->h_state), "arena hipHostFree");
@@ -487,6 +502,8 @@ static int derive_now(anni_adam *opt)
 	if (launch_derive(st, f) != 0)
 		return -1;
 	if (pv->fp8_twins) {
+		if (launch_amax_fold(st, f, nullptr) != 0)
+			return -1;
 		if (launch_fp8_twins(st, f, (uint8_t *)opt->d_param_fp8, opt->d_wscale,
 		    pv->d_wamax[pv->der_cur], pv->d_wamax[pv->der_cur ^ 1], opt->n_tensors,
 		    nullptr) != 0)
@@ -514,7 +531,7 @@ int anni_adam_enable_derived(anni_adam *opt, const anni_pack *packs, int n_packs
 	std::vector<PackDesc> descs;
 	std::vector<Seg> segs;
 	std::vector<float> ones;
-	size_t off_q, off_scale, off_amax, off_packs, off_pack, total;
+	size_t off_q, off_scale, off_amax, off_packs, off_tamax, off_pack, total;
 	char *base;
 	bool fp8 = false;
 
@@ -553,12 +570,19 @@ int anni_adam_enable_derived(anni_adam *opt, const anni_pack *packs, int n_packs
 	off_scale = round_up(fp8 ? (size_t)opt->n : 0, 256);
 	off_amax = off_scale + round_up((size_t)opt->n_tensors * sizeof(float), 256);
 	off_packs = off_amax + 2 * round_up((size_t)opt->n_tensors * sizeof(uint32_t), 256);
-	off_pack = round_up(off_packs + (size_t)opt->n_tensors * sizeof(PackDesc), (size_t)2 << 20);
+	off_tamax = round_up(off_packs + (size_t)opt->n_tensors * sizeof(PackDesc), 256);
+	off_pack = round_up(off_tamax + (fp8 ? (size_t)((opt->n + kTile - 1) / kTile) * kWaves
+	    * sizeof(float) : 0), (size_t)2 << 20);
 	total = off_pack + round_up((size_t)pack_elems * 2, 256) + 256;
-	if (hipMalloc(&pv->derived, total) != hipSuccess) {
+	if (pv->hole && total <= pv->hole_bytes) {
+		pv->derived = pv->hole;
+		pv->derived_owned = 0;
+	} else if (hipMalloc(&pv->derived, total) != hipSuccess) {
 		(void)hipGetLastError();
 		pv->derived = nullptr;
 		return -1;
+	} else {
+		pv->derived_owned = 1;
 	}
 	base = (char *)pv->derived;
 	st = compute_stream();
@@ -567,6 +591,7 @@ int anni_adam_enable_derived(anni_adam *opt, const anni_pack *packs, int n_packs
 	pv->d_wamax[1] = (uint32_t *)(base + off_amax
 	    + round_up((size_t)opt->n_tensors * sizeof(uint32_t), 256));
 	pv->d_packs = (PackDesc *)(base + off_packs);
+	pv->d_tile_amax = fp8 ? (float *)(base + off_tamax) : nullptr;
 	pv->der_cur = 0;
 	pv->fp8_twins = fp8 ? 1 : 0;
 	if (launch_fill_bytes(st, base, 0, total) != 0
@@ -577,7 +602,8 @@ int anni_adam_enable_derived(anni_adam *opt, const anni_pack *packs, int n_packs
 	    || !hip_ok(hipMemcpyAsync(pv->d_segs, segs.data(), (size_t)opt->n_tensors * sizeof(Seg),
 	    hipMemcpyHostToDevice, st), "segs")
 	    || !hip_ok(hipStreamSynchronize(st), "derived init")) {
-		(void)hipFree(pv->derived);
+		if (pv->derived_owned)
+			(void)hipFree(pv->derived);
 		pv->derived = nullptr;
 		return -1;
 	}
@@ -622,6 +648,7 @@ static void describe(const anni_adam *opt, Flat *f)
 	f->gscale = opt->d_gscale;
 	if (pv->derived) {
 		f->der.wamax = pv->fp8_twins ? pv->d_wamax[pv->der_cur] : nullptr;
+		f->der.tile_amax = pv->d_tile_amax;
 		f->der.packs = pv->d_packs;
 		f->der.pack = (uint16_t *)opt->d_pack_bf16;
 	}
@@ -681,6 +708,8 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 	if (ev)
 		(void)hipEventRecord(ev[2], st);
 	if (pv->fp8_twins) {
+		if (launch_amax_fold(st, f, norm.use_norm ? pv->d_state : nullptr) != 0)
+			return -1;
 		if (launch_fp8_twins(st, f, (uint8_t *)opt->d_param_fp8, opt->d_wscale,
 		    pv->d_wamax[pv->der_cur], pv->d_wamax[pv->der_cur ^ 1], opt->n_tensors,
 		    norm.use_norm ? pv->d_state : nullptr) != 0)

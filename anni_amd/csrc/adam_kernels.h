@@ -28,6 +28,7 @@ constexpr int kThreads = 256;			/* four 64-lane wavefronts */
 constexpr int kQuad = 4;			/* elements per lane per access */
 constexpr int kTile = 4096;			/* elements per tile */
 constexpr int kQuadsPerTile = kTile / (kThreads * kQuad);	/* 4 */
+constexpr int kWaves = kThreads / 64;
 constexpr int kMaxPartials = 8192;		/* upper bound on the sum-of-squares grid */
 
 constexpr uint32_t kSegDecay = 1u;		/* decoupled weight decay applies */
@@ -54,11 +55,16 @@ struct PackDesc {
 };
 
 /*
-** Outputs derived from the new weights in the same pass (all NULL: none).  wamax[s] receives
-** max |p| of tensor s as unsigned bits through atomic max (order independent, so deterministic).
+** Outputs derived from the new weights in the same pass (all NULL: none).  Max |p| of the
+** tensors flagged kSegFp8Twin: every wavefront leaves the maximum of its quarter of a whole tile
+** in tile_amax[tile * kWaves + wave] (a plain store; tens of thousands of wavefronts raising
+** one word per tensor were measured to cost the update 3-7 %), the few elements of tiles that
+** straddle tensors raise wamax[s] directly, and launch_amax_fold folds the tile maxima into
+** wamax.  A maximum does not depend on the order, so the result is deterministic.
 */
 struct Derived {
 	uint32_t	*wamax;
+	float		*tile_amax;	/* kWaves floats per tile of the flat */
 	const PackDesc	*packs;		/* one per tensor, read for tensors flagged kSegPack */
 	uint16_t	*pack;
 };
@@ -115,6 +121,12 @@ int	launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double gra
 ** wamax and the packed matrices as the update would leave them.
 */
 int	launch_derive(hipStream_t st, const Flat &f);
+/*
+** wamax[s] = max(wamax[s], tile maxima of tensor s) for the flagged tensors, after
+** launch_update or launch_derive on the same stream.  state (may be NULL): nothing to do
+** after a skipped step.
+*/
+int	launch_amax_fold(hipStream_t st, const Flat &f, const StepState *state);
 /*
 ** q = E4M3(p * (1 / scale_s)) for the tensors flagged kSegFp8Twin, scale_s from wamax[s]
 ** (num/gpu_cuda.cu:826-851,927-938); wscale[s] receives the scale, wamax_next[0..n_tensors) is

@@ -542,8 +542,8 @@ __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 			}
 			if (fp8w) {
 				amax_l = wave_max(amax_l);
-				if ((tid & 63) == 0 && amax_l > 0.0f)
-					amax_raise(a.der.wamax + s, amax_l);
+				if ((tid & 63) == 0)
+					a.der.tile_amax[tile * kWaves + (tid >> 6)] = amax_l;
 			}
 		} else {
 			for (int64_t i = base + tid; i < end; i += kThreads) {
@@ -625,8 +625,8 @@ __global__ __launch_bounds__(kThreads) void derive_kernel(DeriveArgs a)
 			}
 			if (fp8w) {
 				amax_l = wave_max(amax_l);
-				if ((tid & 63) == 0 && amax_l > 0.0f)
-					amax_raise(a.der.wamax + s, amax_l);
+				if ((tid & 63) == 0)
+					a.der.tile_amax[tile * kWaves + (tid >> 6)] = amax_l;
 			}
 		} else {
 			for (int64_t i = base + tid; i < end; i += kThreads) {
@@ -645,6 +645,54 @@ __global__ __launch_bounds__(kThreads) void derive_kernel(DeriveArgs a)
 					pack_one(a.der.pack, a.der.packs[s], (uint32_t)(i - a.segs[s].begin), x);
 			}
 		}
+	}
+}
+
+struct FoldArgs {
+	int64_t		n;
+	const Seg	*segs;
+	const int32_t	*tile_seg;
+	const float	*tile_amax;
+	uint32_t	*wamax;
+	const StepState	*state;
+};
+
+/*
+** One lane per tile: the four wavefront maxima of a whole tile of a flagged tensor (the tiles
+** the vector paths above wrote) go into the tensor's word.  Neighbouring tiles mostly belong
+** to one tensor, so a wavefront whose 64 tiles all do raises the word once.
+*/
+__global__ __launch_bounds__(kThreads) void amax_fold_kernel(FoldArgs a)
+{
+	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
+	const int64_t tile = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+	int s = -1;
+	float mx = 0.0f;
+
+	if (a.state != nullptr && a.state->skipped != 0)
+		return;
+	if (tile < n_tiles) {
+		const int t = a.tile_seg[tile];
+		const int64_t base = tile * kTile;
+
+		if (base + kTile <= a.n && a.segs[t].end >= base + kTile
+		    && (a.segs[t].flags & kSegFp8Twin) != 0) {
+			const f32x4 w = *(const f32x4 *)(a.tile_amax + tile * kWaves);
+
+			s = t;
+			mx = fmaxf(fmaxf(w.x, w.y), fmaxf(w.z, w.w));
+		}
+	}
+	const int s0 = __shfl(s, 0, 64);
+
+	if (__all(s == s0)) {
+		if (s0 < 0)
+			return;
+		mx = wave_max(mx);
+		if ((threadIdx.x & 63) == 0 && mx > 0.0f)
+			amax_raise(a.wamax + s0, mx);
+	} else if (s >= 0 && mx > 0.0f) {
+		amax_raise(a.wamax + s, mx);
 	}
 }
 
@@ -979,6 +1027,8 @@ static int check_derived(const Flat &f)
 		return 0;
 	if (!f.segs || !f.tile_seg)
 		return -1;
+	if (f.der.wamax && !aligned(f.der.tile_amax, 16))
+		return -1;
 	if (f.der.pack && (!f.der.packs || !aligned(f.der.pack, 8)))
 		return -1;
 	return 0;
@@ -1008,6 +1058,8 @@ int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double gra
 	a.vec_ok = aligned(f.p, 16) && aligned(f.g, quad_bytes(f.grad_type))
 	    && aligned(f.m, quad_bytes(f.moment_type)) && aligned(f.v, quad_bytes(f.moment_type))
 	    && (!f.twin || aligned(f.twin, 8)) ? 1 : 0;
+	if (f.der.wamax && !a.vec_ok)
+		return -1;	/* the tile maxima come from the vector path: the flats must be aligned */
 	a.c = c;
 	a.grad_scale = grad_scale;
 	a.use_norm = norm.use_norm;
@@ -1068,10 +1120,31 @@ int launch_derive(hipStream_t st, const Flat &f)
 	a.tile_seg = f.tile_seg;
 	a.der = f.der;
 	a.vec_ok = aligned(f.p, 16) ? 1 : 0;
+	if (f.der.wamax && !a.vec_ok)
+		return -1;
 	if (nt_on())
 		hipLaunchKernelGGL((derive_kernel<true>), dim3(grid_for(f.n)), dim3(kThreads), 0, st, a);
 	else
 		hipLaunchKernelGGL((derive_kernel<false>), dim3(grid_for(f.n)), dim3(kThreads), 0, st, a);
+	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int launch_amax_fold(hipStream_t st, const Flat &f, const StepState *state)
+{
+	FoldArgs a;
+	const int64_t n_tiles = (f.n + kTile - 1) / kTile;
+
+	static_assert(kWaves == 4, "one 16-byte load per tile");
+	if (f.n <= 0 || !f.der.wamax || check_derived(f) != 0)
+		return -1;
+	a.n = f.n;
+	a.segs = f.segs;
+	a.tile_seg = f.tile_seg;
+	a.tile_amax = f.der.tile_amax;
+	a.wamax = f.der.wamax;
+	a.state = state;
+	hipLaunchKernelGGL(amax_fold_kernel, dim3((unsigned)((n_tiles + kThreads - 1) / kThreads)),
+	    dim3(kThreads), 0, st, a);
 	return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

@@ -223,6 +223,10 @@ def main():
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="only run the plain copy kernel over BYTES ten times (counter calibration)")
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds for the CPU legs")
+    ap.add_argument("--derived", nargs="?", const="both", default=None,
+                    choices=["both", "fp8", "pack"],
+                    help="the reference's own tensor list (separate Wq, Wk, Wv) with the fused "
+                         "producers on: E4M3 twins of every matrix and a packed [Wq|Wk|Wv] per block")
     ap.add_argument("--ref-jsonl", default=None, metavar="FILE",
                     help="also append one row in the reference's bench-log schema (optimizer "
                          "phase only); steps are then timed one call each")
@@ -247,13 +251,29 @@ def main():
         return
 
     size, gt, mt, norm_bpp, upd_bpp = WORKLOADS[a.workload]
-    tensors = layout.tensors(size)
+    tensors = layout.tensors(size, "reference" if a.derived else "baseline")
+    packs, pack_elems, fp8_elems = [], 0, 0
+    if a.derived:
+        if gt != 0 or mt != 0:
+            sys.exit("bench.py: --derived is measured on the all-f32 workloads")
+        d = layout.SIZES[size][0]
+        names = [t[0] for t in tensors]
+        if a.derived != "pack":
+            tensors = [(nm, cnt, f | (lib.T_FP8TWIN if f & lib.T_TWIN else 0))
+                       for nm, cnt, f in tensors]
+        fp8_elems = sum(cnt for _nm, cnt, f in tensors if f & lib.T_FP8TWIN)
+        for b in range(layout.SIZES[size][3] if a.derived != "fp8" else 0):
+            for k, w in enumerate(("wq", "wk", "wv")):
+                packs.append((names.index("blk%d.%s" % (b, w)), d, pack_elems + k * d, 3 * d))
+            pack_elems += 3 * d * d
     total = a.steps + a.warmup
     opt = LmAdam(tensors, grad_type=gt, moment_type=mt, twins=True, skip_nonfinite=True,
                  grad_slots=total, layout={"auto": 0, "compact": 1, "spread": 2}[a.layout],
                  beta2=0.95, weight_decay=0.1, grad_clip=1.0)
     n = opt.n
     assert L.anni_fill_normal_f32(opt.o.d_param, n, 20260101, 1, 0.0, 0.02) == 0
+    if a.derived:
+        opt.enable_derived(packs, pack_elems)
     opt.seed_twins()
     ring, scales = fill_grad_slots(L, opt, tensors, total, gt, 20260101)
 
@@ -312,10 +332,14 @@ def main():
     assert opt.t == total and math.isfinite(st.last_grad_norm)
     bpp = norm_bpp + upd_bpp
     ms_step = wall_ms / a.steps
-    step_gbps = n * bpp / (ms_step * 1e-3) / 1e9
+    # derived outputs: 2 more bytes written per packed element by the update, and the E4M3 pass
+    # reads p (4) and writes the code (1) of every flagged element
+    extra_bytes = 2 * pack_elems + 5 * fp8_elems
+    step_gbps = (n * bpp + extra_bytes) / (ms_step * 1e-3) / 1e9
     upd_ms = ms_update / a.steps
     sumsq_ms = ms_sumsq / a.steps
-    upd_gbps = n * upd_bpp / (upd_ms * 1e-3) / 1e9
+    upd_bytes = n * upd_bpp + 2 * pack_elems
+    upd_gbps = upd_bytes / (upd_ms * 1e-3) / 1e9
     out = {
         "metric": "AdamW step HBM GB/s (algorithmic bytes / step time; AdamW + global-norm clip "
                   "+ decay + bf16 twins), %s param set" % a.workload,
@@ -335,13 +359,26 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "adam_update_kernel", "achieved": round(upd_gbps, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(upd_gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": TRAFFIC_BYTES.get(a.workload),
-                     "bytes_per_launch": n * upd_bpp, "avg_ms": round(upd_ms, 4)},
+                     "traffic": None if a.derived else TRAFFIC_BYTES.get(a.workload),
+                     "bytes_per_launch": upd_bytes, "avg_ms": round(upd_ms, 4)},
         "sumsq_kernel": {"avg_ms": round(sumsq_ms, 4), "bytes_per_launch": n * norm_bpp,
                          "achieved": round(n * norm_bpp / (sumsq_ms * 1e-3) / 1e9, 1)
                          if sumsq_ms > 0 else None, "unit": "GB/s"},
         "last_grad_norm": st.last_grad_norm, "last_clipped": int(st.last_clipped),
     }
+    if a.derived:
+        der_ms = L.anni_adam_timed_derived_ms(opt.h) / a.steps
+        out["config"]["derived"] = {"both": "E4M3 twins of every matrix + packed [Wq|Wk|Wv] per block",
+                                    "fp8": "E4M3 twins of every matrix",
+                                    "pack": "packed [Wq|Wk|Wv] per block"}[a.derived]
+        out["config"]["launches_per_step"] = 3 if fp8_elems else 2
+        out["derived"] = {
+            "fp8_twin_kernel": {"avg_ms": round(der_ms, 4), "bytes_per_launch": 5 * fp8_elems,
+                                "achieved": round(5 * fp8_elems / (der_ms * 1e-3) / 1e9, 1)
+                                if der_ms > 0 else None, "unit": "GB/s"},
+            "fp8_twin_elems": fp8_elems, "packed_elems": pack_elems,
+            "separate_passes_would_move_bytes": 9 * fp8_elems + 4 * pack_elems,
+            "fused_moves_bytes": extra_bytes}
     if not a.no_cpu:
         mt_out, serial_out = cpu_baselines(size, norm_bpp, upd_bpp, a.cpu_budget)
         out["cpu_baseline"] = mt_out

@@ -209,3 +209,51 @@ def test_refusals(gpu):
     assert enable([(0, 64, 0, 64)], 4096) == 0
     assert enable([(0, 64, 0, 64)], 4096) == -1                   # once only
     opt.free()
+
+
+def test_185m_reference_layout_full_size(gpu, oracle):
+    """The reference's own model size (separate Wq, Wk, Wv of 1024 x 1024, 12 blocks): E4M3 twins of
+    all 74 matrices and the 12 packed [1024][3072] operands over two steps, one of them clipped,
+    every element compared."""
+    import math
+    import os
+    from anni_amd import layout
+    threads = max(1, min(16, len(os.sched_getaffinity(0))))
+    d, _h, _ff, blocks, _v = layout.SIZES["185m"]
+    tensors = [(name, n, f | (FP8TWIN if f & TWIN else 0))
+               for name, n, f in layout.tensors("185m", "reference")]
+    names = [t[0] for t in tensors]
+    packs, pack_elems = [], 0
+    for b in range(blocks):
+        for k, w in enumerate(("wq", "wk", "wv")):
+            packs.append((names.index("blk%d.%s" % (b, w)), d, pack_elems + k * d, 3 * d))
+        pack_elems += 3 * d * d
+    opt = make(tensors, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True)
+    n = opt.n
+    assert gpu.anni_fill_normal_f32(opt.o.d_param, n, 4, 1, 0.0, 0.02) == 0
+    opt.enable_derived(packs, pack_elems)
+    opt.seed_twins()
+    P = opt.download("param")
+    M, V = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    q, sc = want_fp8(oracle, opt, P, np.zeros(n, np.uint8), np.ones(len(tensors), np.float32))
+    pk = want_pack(oracle, opt, P, packs, pack_elems, np.zeros(pack_elems, np.uint16))
+    assert (opt.download("fp8twin") == q).all() and same_bits(opt.download("wscale"), sc)
+    assert (opt.download("pack") == pk).all()
+    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True,
+                      tensors=oracle_tensors(opt), threads=threads, simd=oracle.cpu_simd())
+    unit = 1.0 / (math.sqrt(n) * 1e-3)
+    for s, mult in enumerate((1.7, 0.6)):
+        assert gpu.anni_fill_normal_f32(opt.o.d_grad, n, 4, 50 + s, 0.0, 1e-3) == 0
+        g = opt.download("grad")
+        assert opt.step_scaled(3e-4, unit * mult) == 0
+        st = opt.sync_stats()
+        assert st.last_clipped == (mult > 1)
+        O.step(P, g, M, V, 3e-4, unit * mult, sumsq_override=st.last_sumsq)
+        assert same_bits(opt.download("param"), P)
+        q, sc = want_fp8(oracle, opt, P, q, sc)
+        pk = want_pack(oracle, opt, P, packs, pack_elems, pk)
+        assert (opt.download("fp8twin") == q).all(), s
+        assert same_bits(opt.download("wscale"), sc), s
+        assert (opt.download("pack") == pk).all(), s
+        print("185m derived step %d ok" % (s + 1), flush=True)
+    opt.free()
