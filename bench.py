@@ -30,10 +30,10 @@ HBM_PEAK_GBPS = 8000.0
 
 # name: (size, grad_type, moment_type, bytes/param of the norm pass, bytes/param of the update)
 WORKLOADS = {
-    "185m": ("185m", 0, 0, 4, 34),          # BASELINE config 2
-    "555m": ("555m", 0, 0, 4, 34),          # BASELINE config 3 (headline)
-    "555m-bf16": ("555m", 1, 1, 2, 22),     # BASELINE config 4
-    "1p4b-fp8": ("1p4b", 2, 0, 1, 28),      # BASELINE config 5
+    "185m": ("185m", 0, 0, 4, 34),          # benchmark configuration 2
+    "555m": ("555m", 0, 0, 4, 34),          # benchmark configuration 3 (headline)
+    "555m-bf16": ("555m", 1, 1, 2, 22),     # benchmark configuration 4
+    "1p4b-fp8": ("1p4b", 2, 0, 1, 28),      # benchmark configuration 5
     "1p4b": ("1p4b", 0, 0, 4, 34),          # the 1.4B set in the all-f32 mode (comparison only)
 }
 ELEM = {0: 4, 1: 2, 2: 1}

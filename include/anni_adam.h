@@ -52,7 +52,7 @@ extern "C" {
 #define ANNI_LAYOUT_SPREAD	2
 
 /* Tensor flags. */
-#define ANNI_T_DECAY	1u	/* decoupled weight decay applies (BASELINE: matrices only) */
+#define ANNI_T_DECAY	1u	/* decoupled weight decay applies (the benchmark configurations: matrices only) */
 #define ANNI_T_TWIN	2u	/* the bf16 twin of this tensor is written */
 #define ANNI_T_FP8TWIN	4u	/* an E4M3 twin with its own scale is kept current (needs anni_adam_enable_derived) */
 

@@ -294,6 +294,8 @@ def _declare_model(R):
     R.ref_model_load_checkpoint.argtypes = [C.c_char_p, C.POINTER(C.c_int), C.POINTER(C.c_int)]
     R.ref_model_load_checkpoint.restype = C.c_void_p
     R.ref_model_free.argtypes = [C.c_void_p]
+    R.ref_set_offload.argtypes = [C.c_int]
+    R.ref_model_mv_on_device.argtypes = [C.c_void_p]
 
 
 _ref_cpu_model = None
@@ -376,6 +378,14 @@ class RefModelOnBackend:
     @property
     def last_grad_norm(self):
         return self.R.ref_model_last_norm(self.h)
+
+    def set_offload(self, on):
+        """lm_adam_set_offload: a process-wide switch of the reference."""
+        self.R.ref_set_offload(int(on))
+
+    @property
+    def mv_on_device(self):
+        return bool(self.R.ref_model_mv_on_device(self.h))
 
     def close(self):
         if self.h:

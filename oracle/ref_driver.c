@@ -233,6 +233,17 @@ int ref_model_set_grads(ref_model *r, const float *flat)
 	return 0;
 }
 
+/* lm_adam_set_offload (lang/lm_adam.c:211-214): m and v leave the device after every step. */
+void ref_set_offload(int on)
+{
+	lm_adam_set_offload(on);
+}
+
+int ref_model_mv_on_device(const ref_model *r)
+{
+	return r->opt->d_m != NULL && r->opt->d_v != NULL;
+}
+
 int ref_model_step(ref_model *r, double lr, double grad_scale)
 {
 	lm_adam_step_scaled(r->opt, lr, grad_scale);

@@ -25,10 +25,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 STEPS = 10
 
 CASES = {
-    # BASELINE config 1: constant lr 3e-4, no clip, wd 0.1, beta2 0.95
+    # benchmark configuration 1: constant lr 3e-4, no clip, wd 0.1, beta2 0.95
     "cfg1_noclip": dict(n=1531, seed=11, base_lr=3e-4, sched=None, wd=0.1, clip=0.0,
                         beta2=0.95, gmul=[1.0] * STEPS, grad_scale=1.0),
-    # BASELINE config 2: clip 1.0 with about half the steps clipping, warmup 100 + cosine
+    # benchmark configuration 2: clip 1.0 with about half the steps clipping, warmup 100 + cosine
     "cfg2_clip_sched": dict(n=1531, seed=12, base_lr=3e-4, sched=(100, 1000, "cosine"),
                             wd=0.1, clip=1.0, beta2=0.95,
                             gmul=[13.0, 40.0, 20.0, 70.0, 8.0, 33.0, 52.0, 18.0, 25.0, 61.0],

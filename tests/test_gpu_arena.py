@@ -1,5 +1,5 @@
 """Parity of the multi-tensor arena step (include/anni_adam.h) against the CPU oracle, through the
-C ABI: BASELINE configurations at reduced size, ragged tensor lists, every storage mode, the
+C ABI: the benchmark configurations at reduced size, ragged tensor lists, every storage mode, the
 non-finite skip, and the golden vectors of the reference."""
 import numpy as np
 import pytest
@@ -8,8 +8,8 @@ from helpers import GOLDEN_CASES, load_golden, same_bits, rel_err, bf16_ulp_diff
 
 pytestmark = pytest.mark.gpu
 
-TOL_STATE = 1e-6     # BASELINE: FP32 master/m/v within 1e-6 relative per step
-TOL_NORM = 1e-5      # BASELINE: clip norm within 1e-5 relative
+TOL_STATE = 1e-6     # required: FP32 master/m/v within 1e-6 relative per step
+TOL_NORM = 1e-5      # required: clip norm within 1e-5 relative
 
 F32, BF16, FP8 = 0, 1, 2
 DECAY, TWIN = 1, 2
@@ -42,7 +42,7 @@ def twin_mask(opt):
 def run_fp32_case(gpu, oracle, tensors, steps, clip, wd, gmul, grad_scale=1.0, seed=0,
                   sched=(100, 1000, "cosine"), layout=0):
     """Ten steps on the arena vs the oracle twice: against the oracle's own (serial) norm with the
-    BASELINE tolerances, and bit for bit when the oracle is handed the device's sum of squares."""
+    required tolerances, and bit for bit when the oracle is handed the device's sum of squares."""
     from anni_amd import lm_adam
     rng = np.random.default_rng(seed)
     opt = make(gpu, tensors, beta2=0.95, weight_decay=wd, grad_clip=clip, layout=layout)
@@ -105,12 +105,12 @@ def test_spread_layout_gives_the_same_results(gpu, oracle):
 
 
 def test_config1_no_clip_ragged(gpu, oracle):
-    """BASELINE config 1 hyper-parameters (constant lr, no clip, decay on flagged tensors)."""
+    """benchmark configuration 1 hyper-parameters (constant lr, no clip, decay on flagged tensors)."""
     run_fp32_case(gpu, oracle, RAGGED, 10, clip=0.0, wd=0.1, gmul=[1.0], sched=(0, 0, "none"))
 
 
 def test_config2_clip_half_the_steps_ragged(gpu, oracle):
-    """BASELINE config 2: clip 1.0 with about half the steps clipping, warmup 100 + cosine."""
+    """benchmark configuration 2: clip 1.0 with about half the steps clipping, warmup 100 + cosine."""
     n = sum(t[0] for t in RAGGED)
     base = 1.0 / (np.sqrt(n) * 1e-3)                       # gmul = base -> norm ~ 1
     k = run_fp32_case(gpu, oracle, RAGGED, 10, clip=1.0, wd=0.1,
@@ -210,7 +210,7 @@ def test_without_skip_flag_nonfinite_poisons_like_the_cpu_path(gpu, oracle):
 
 
 def test_bf16_moments_and_grads(gpu, oracle):
-    """BASELINE config 4 at reduced size, long tail included (parity unpinned by the reference:
+    """benchmark configuration 4 at reduced size, long tail included (parity unpinned by the reference:
     the oracle defines the rounding points)."""
     rng = np.random.default_rng(44)
     opt = make(gpu, RAGGED, grad_type=BF16, moment_type=BF16, beta2=0.95, weight_decay=0.1,
@@ -247,7 +247,7 @@ def test_bf16_moments_and_grads(gpu, oracle):
 
 
 def test_fp8_gradients_with_per_tensor_scale_and_skip(gpu, oracle):
-    """BASELINE config 5 at reduced size: device quantisation, in-kernel unscale, NaN skip."""
+    """benchmark configuration 5 at reduced size: device quantisation, in-kernel unscale, NaN skip."""
     rng = np.random.default_rng(55)
     tensors = [(6000, 3), (64, 0), (4096, 3), (8192 + 3, 3), (1, 0), (20000, 3)]
     opt = make(gpu, tensors, grad_type=FP8, beta2=0.95, weight_decay=0.1, grad_clip=1.0,

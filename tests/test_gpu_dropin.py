@@ -1,6 +1,6 @@
 """Parity of the flat drop-in ABI (the num/gpu.h entry points lang/lm_adam.c calls) against the
 CPU oracle, through the C ABI.  Bit-exact where the arithmetic is identical by construction;
-BASELINE tolerances (1e-6 relative on p/m/v, 1 bf16 ulp on twins, 1e-5 on the norm) where the
+required tolerances (1e-6 relative on p/m/v, 1 bf16 ulp on twins, 1e-5 on the norm) where the
 summation order of the norm differs."""
 import ctypes as C
 import math
@@ -12,8 +12,8 @@ from helpers import GOLDEN_CASES, load_golden, same_bits, rel_err, bf16_ulp_diff
 
 pytestmark = pytest.mark.gpu
 
-TOL_STATE = 1e-6     # BASELINE: FP32 master/m/v within 1e-6 relative per step
-TOL_NORM = 1e-5      # BASELINE: clip norm within 1e-5 relative
+TOL_STATE = 1e-6     # required: FP32 master/m/v within 1e-6 relative per step
+TOL_NORM = 1e-5      # required: clip norm within 1e-5 relative
 
 
 def dev(gpu, arr):
@@ -232,7 +232,7 @@ def reference_device_flow(gpu, S, t, lr, grad_scale, clip, wd):
 
 
 def test_unchanged_caller_flow_matches_cpu_path(gpu, oracle):
-    """What lang/lm_adam.c does with this backend vs its own host loop: BASELINE tolerances.
+    """What lang/lm_adam.c does with this backend vs its own host loop: required tolerances.
     (The caller's device branch scales by clip/norm, its host loop by clip/(norm+1e-12).)"""
     n = 300007
     S = FlatState(gpu, n, seed=5)

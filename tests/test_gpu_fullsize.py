@@ -1,4 +1,4 @@
-"""The BASELINE configurations at their real sizes on the GPU, against the CPU oracle run on the
+"""The benchmark configurations at their real sizes on the GPU, against the CPU oracle run on the
 host cores of the same box (multithreaded, bit-identical per element to the serial loop) and
 through size-independent properties.  Data are generated on the device and copied down once."""
 import ctypes as C
@@ -12,8 +12,8 @@ from helpers import same_bits, rel_err, bf16_ulp_diff
 
 pytestmark = pytest.mark.gpu
 
-TOL_STATE = 1e-6     # BASELINE: FP32 master/m/v within 1e-6 relative per step over 10 steps
-TOL_NORM = 1e-5      # BASELINE: clip norm within 1e-5 relative
+TOL_STATE = 1e-6     # required: FP32 master/m/v within 1e-6 relative per step over 10 steps
+TOL_NORM = 1e-5      # required: clip norm within 1e-5 relative
 THREADS = max(1, min(16, len(os.sched_getaffinity(0))))
 
 
@@ -34,7 +34,7 @@ def setup(gpu, size, **kw):
 
 
 def test_config2_185m_ten_steps(gpu, oracle):
-    """BASELINE config 2 as stated: 185M set, clip 1.0 with half the steps clipping, warmup 100 +
+    """benchmark configuration 2 as stated: 185M set, clip 1.0 with half the steps clipping, warmup 100 +
     cosine at steps 1..10, decay on matrices only, twins of every matrix; 10 steps, every step
     compared on all 167,948,288 parameters."""
     from anni_amd import lm_adam
@@ -85,7 +85,7 @@ def checksum(gpu, ptr, n):
 
 
 def test_config3_555m_step_and_properties(gpu, oracle):
-    """BASELINE config 3 (headline): two full steps compared bit for bit on all 555,848,096
+    """benchmark configuration 3 (headline): two full steps compared bit for bit on all 555,848,096
     parameters, then size-independent properties of a skipped and a clipped step."""
     opt, tensors, segs, mask = setup(gpu, "555m", skip_nonfinite=True)
     n = opt.n
@@ -130,7 +130,7 @@ def test_config3_555m_step_and_properties(gpu, oracle):
 
 
 def test_config4_555m_bf16_moments_and_grads(gpu, oracle):
-    """BASELINE config 4: bf16-stored m/v, bf16 gradients, long tail of tiny tensors; one full
+    """benchmark configuration 4: bf16-stored m/v, bf16 gradients, long tail of tiny tensors; one full
     step bit for bit (parity unpinned by the reference: the oracle defines the rounding points)."""
     opt, tensors, segs, mask = setup(gpu, "555m", grad_type=1, moment_type=1)
     n = opt.n
@@ -159,7 +159,7 @@ def test_config4_555m_bf16_moments_and_grads(gpu, oracle):
 
 
 def test_config5_1p4b_fp8_grads_and_nan_skip(gpu, oracle):
-    """BASELINE config 5: 1.4B set, fp8-e4m3 gradients with a per-tensor scale from the tensor's
+    """benchmark configuration 5: 1.4B set, fp8-e4m3 gradients with a per-tensor scale from the tensor's
     amax, unscaled in the kernel; one seeded step carries a NaN in one tensor and must leave the
     state bit-identical; the normal step is compared bit for bit on all 1,413,498,528 parameters."""
     opt, tensors, segs, mask = setup(gpu, "1p4b", grad_type=2, skip_nonfinite=True)
@@ -263,3 +263,47 @@ def test_reference_production_flow_on_this_backend(gpu, oracle):
     M.close()
     gpu.gpu_set_compute_prec(0)
     gpu.gpu_adam_set_weight_decay(0.0)
+
+
+def test_reference_offload_between_steps_on_this_backend(gpu, oracle):
+    """lm_adam_set_offload(1) (lang/lm_adam.c:211-214,296-345): after every step the unchanged
+    caller reads m and v back, frees their device flats and allocates and uploads them again for
+    the next one -- repeated gpu_free / gpu_malloc of 600 MB blocks next to the live p, g and twin
+    flats.  Results must not change: three steps against the oracle, every element."""
+    if not oracle.ref_hip_available():
+        pytest.skip("oracle/_ref/libanni_ref_hip.so not built (reference tree absent at build time)")
+    gpu.gpu_set_compute_prec(1)
+    M = oracle.RefModelOnBackend(64, beta2=0.95, weight_decay=0.1, grad_clip=1.0)
+    n = M.n
+    P = M.params()
+    Mo, Vo = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, threads=THREADS, simd=oracle.cpu_simd())
+    rng = np.random.default_rng(6)
+    unit = 1.0 / (math.sqrt(n) * 1e-3)
+    fr0, tt = C.c_size_t(0), C.c_size_t(0)
+    try:
+        M.set_offload(1)
+        for t in range(1, 4):
+            g = rng.standard_normal(n, dtype=np.float32) * np.float32(1e-3)
+            M.set_grads(g)
+            lr = oracle.lr(3e-4, t - 1, 100, 1000, "cosine")
+            gs = unit * (1.7 if t % 2 else 0.6)
+            assert M.step(lr, gs) == t and M.on_device
+            assert not M.mv_on_device                      # offloaded after the step
+            norm = M.last_grad_norm
+            O.step(P, g, Mo, Vo, lr, gs * (1.0 / norm) if norm > 1.0 else gs)
+            fr = C.c_size_t(0)
+            assert gpu.gpu_mem_info(C.byref(fr), C.byref(tt)) == 0
+            if t == 1:
+                fr0 = fr
+            assert fr.value == fr0.value, "device memory in use moved between steps"
+            print("offload step %d ok (norm %.4f)" % (t, norm), flush=True)
+        M.set_offload(0)
+        p = M.params()
+        m, v = M.moments()
+        assert same_bits(p, P) and same_bits(m, Mo) and same_bits(v, Vo)
+    finally:
+        M.set_offload(0)
+        M.close()
+        gpu.gpu_set_compute_prec(0)
+        gpu.gpu_adam_set_weight_decay(0.0)
