@@ -270,8 +270,7 @@ static int g_pinned_n;
 
 /* Scratch of the flat path: sum-of-squares partials + the step state, and a pinned result word. */
 static double *g_partials;
-static StepState *g_state;
-static double *g_host_result;
+static StepState *g_host_state;		/* page-locked, written by the device */
 
 static bool scratch_ready(void)
 {
@@ -282,7 +281,7 @@ static bool scratch_ready(void)
 	void *d = nullptr;
 	void *h = nullptr;
 
-	if (hipMalloc(&d, sizeof(double) * kMaxPartials + sizeof(StepState)) != hipSuccess
+	if (hipMalloc(&d, sizeof(double) * kMaxPartials) != hipSuccess
 	    || hipHostMalloc(&h, sizeof(StepState), hipHostMallocDefault) != hipSuccess) {
 		(void)hipGetLastError();
 		if (d)
@@ -290,8 +289,8 @@ static bool scratch_ready(void)
 		return false;
 	}
 	g_partials = (double *)d;
-	g_state = (StepState *)(g_partials + kMaxPartials);
-	g_host_result = (double *)h;
+	g_host_state = (StepState *)h;
+	memset(g_host_state, 0, sizeof(*g_host_state));
 	return true;
 }
 
@@ -742,15 +741,14 @@ int gpu_grad_sumsq(const ann_real *d_x, int n, double *out)
 	{
 		ProfScope prof(0);
 
+		/* the one-workgroup second stage stores its result straight into page-locked host memory */
 		if (launch_sumsq(g_stream, f, 1.0, g_partials, &np) != 0
-		    || launch_finalize(g_stream, g_partials, np, 0.0, 0, 1.0, g_state) != 0)
+		    || launch_finalize(g_stream, g_partials, np, 0.0, 0, 1.0, g_host_state) != 0)
 			return -1;
 	}
-	if (!hip_ok(hipMemcpyAsync(g_host_result, &g_state->sumsq, sizeof(double),
-	    hipMemcpyDeviceToHost, g_stream), "sumsq d2h")
-	    || !hip_ok(sync_stream_and_deliver(), "sumsq sync"))
+	if (!hip_ok(sync_stream_and_deliver(), "sumsq sync"))
 		return -1;
-	*out = *g_host_result;
+	*out = g_host_state->sumsq;
 	return 0;
 }
 
