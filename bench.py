@@ -222,6 +222,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="only run the plain copy kernel over BYTES ten times (counter calibration)")
+    ap.add_argument("--reference-caller-only", action="store_true",
+                    help="only time the unchanged reference caller on this backend (one JSON line)")
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds for the CPU legs")
     ap.add_argument("--derived", nargs="?", const="both", default=None,
                     choices=["both", "fp8", "pack"],
@@ -248,6 +250,9 @@ def main():
         env = bench_row.probe_env(L, os.path.dirname(os.path.abspath(__file__)))
     if a.copy_calibration:
         copy_calibration(L, a.copy_calibration)
+        return
+    if a.reference_caller_only:
+        print(json.dumps(reference_caller_leg(L)))
         return
 
     size, gt, mt, norm_bpp, upd_bpp = WORKLOADS[a.workload]
