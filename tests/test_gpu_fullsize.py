@@ -307,3 +307,52 @@ def test_reference_offload_between_steps_on_this_backend(gpu, oracle):
         M.close()
         gpu.gpu_set_compute_prec(0)
         gpu.gpu_adam_set_weight_decay(0.0)
+
+
+@pytest.mark.parametrize("mode", ["f32", "bf16"])
+def test_more_than_2_to_31_elements(gpu, oracle, mode):
+    """64-bit indexing: 2,281,707,523 elements, one tensor ending past 2^31, a tensor list whose
+    offsets do not fit 32 bits.  Closed form instead of a host oracle: p = 1, g = m = v = 0, so
+    the Adam part leaves p alone and the decay gives (float)(1 - lr*wd) = 1 - 2^-10 exactly on the
+    flagged tensors; sums of squares of such values over any slice are exact in double."""
+    from anni_amd.lm_adam import LmAdam
+    tensors = [((1 << 31) - 1000, 3), (5000, 2), ((1 << 27) + 4523, 3)]
+    narrow = 1 if mode == "bf16" else 0
+    opt = LmAdam(tensors, grad_type=narrow, moment_type=narrow, beta2=0.95, weight_decay=0.5,
+                 grad_clip=1.0, skip_nonfinite=True)
+    n = opt.n
+    assert n > (1 << 31) and opt.offsets[2] > (1 << 31) - 1
+    assert gpu.anni_fill_normal_f32(opt.o.d_param, n, 1, 1, 1.0, 0.0) == 0
+    opt.seed_twins()
+    assert opt.step_scaled(2.0 ** -9) == 0                    # lr * wd = 2^-10
+    st = opt.sync_stats()
+    assert st.last_sumsq == 0.0 and st.last_skipped == 0 and st.last_clipped == 0
+    c1 = 1.0 - 2.0 ** -10
+
+    def slices(off, cnt, step=(1 << 30)):
+        while cnt > 0:
+            k = min(cnt, step)
+            yield off, k
+            off, cnt = off + k, cnt - k
+    for (off, cnt, flagged) in ((opt.offsets[0], tensors[0][0], True), (opt.offsets[1], 5000, False),
+                                (opt.offsets[2], tensors[2][0], True)):
+        want = c1 * c1 if flagged else 1.0
+        for o, k in slices(off, cnt):
+            assert checksum(gpu, opt.o.d_param + 4 * o, k) == k * want, (o, k)
+    if mode == "f32":
+        for name in ("m", "v", "grad"):
+            ptr = {"m": opt.o.d_m, "v": opt.o.d_v, "grad": opt.o.d_grad}[name]
+            for o, k in slices(0, n):
+                assert checksum(gpu, ptr + 4 * o, k) == 0.0, name
+    # twins (1 - 2^-10 rounds to 1.0 in bf16) and the state around the places where 32-bit
+    # arithmetic would wrap
+    for at in (0, (1 << 31) - 3000, (1 << 31) - 8, opt.offsets[2] - 100, n - 6000):
+        k = min(6000, n - at)
+        assert (opt.download("twin", k, at) == 0x3f80).all(), at
+        p = opt.download("param", k, at)
+        idx = np.arange(at, at + k)
+        flagged = (idx < opt.offsets[1]) | (idx >= opt.offsets[2])
+        assert (p[flagged] == np.float32(c1)).all() and (p[~flagged] == 1.0).all(), at
+        assert not opt.download("m", k, at).any() and not opt.download("v", k, at).any()
+        assert not opt.download("grad", k, at).any()
+    opt.free()
