@@ -283,8 +283,9 @@ static double probe(const anni_adam *opt)
 
 extern "C" {
 
-anni_adam *anni_adam_create(const anni_tensor *tensors, int n_tensors,
-	const anni_adam_config *cfg)
+/* *made holds the handle as soon as it exists, so the caller can release it if this throws. */
+static anni_adam *create_body(const anni_tensor *tensors, int n_tensors,
+	const anni_adam_config *cfg, anni_adam **made)
 {
 	const size_t big = (size_t)2 << 20;	/* each flat starts on a 2 MiB boundary */
 	/* A spread arena is requested again (up to kTries) while the probe stays below these. */
@@ -323,6 +324,7 @@ anni_adam *anni_adam_create(const anni_tensor *tensors, int n_tensors,
 		return nullptr;
 	}
 	opt->priv = pv;
+	*made = opt;
 	opt->n = n;
 	opt->n_tensors = n_tensors;
 	opt->beta1 = 0.9;	/* lm_adam.c:110-115 */
@@ -371,6 +373,7 @@ anni_adam *anni_adam_create(const anni_tensor *tensors, int n_tensors,
 	if (!hip_ok(hipHostMalloc((void **)&pv->h_state, sizeof(StepState), hipHostMallocDefault),
 	    "arena hipHostMalloc")) {
 		(void)hipGetLastError();
+		*made = nullptr;
 		anni_adam_free(&opt);
 		return nullptr;
 	}
@@ -429,10 +432,27 @@ anni_adam *anni_adam_create(const anni_tensor *tensors, int n_tensors,
 	}
 	if (!ok) {
 		(void)hip_ok(hipErrorOutOfMemory, "arena hipMalloc");
+		*made = nullptr;
 		anni_adam_free(&opt);
 		return nullptr;
 	}
 	return opt;
+}
+
+void anni_adam_free(anni_adam **popt);
+
+/* No C++ exception (a failed host allocation) crosses the C boundary: the answer is NULL / -1. */
+anni_adam *anni_adam_create(const anni_tensor *tensors, int n_tensors,
+	const anni_adam_config *cfg)
+{
+	anni_adam *made = nullptr;
+
+	try {
+		return create_body(tensors, n_tensors, cfg, &made);
+	} catch (...) {
+		anni_adam_free(&made);
+		return nullptr;
+	}
 }
 
 void anni_adam_free(anni_adam **popt)
@@ -523,7 +543,7 @@ int anni_adam_seed_twins(anni_adam *opt)
 	return opt->priv->derived ? derive_now(opt) : 0;
 }
 
-int anni_adam_enable_derived(anni_adam *opt, const anni_pack *packs, int n_packs,
+static int enable_derived_body(anni_adam *opt, const anni_pack *packs, int n_packs,
 	int64_t pack_elems)
 {
 	anni_adam_priv *pv;
@@ -614,6 +634,16 @@ int anni_adam_enable_derived(anni_adam *opt, const anni_pack *packs, int n_packs
 	return 0;
 }
 
+int anni_adam_enable_derived(anni_adam *opt, const anni_pack *packs, int n_packs,
+	int64_t pack_elems)
+{
+	try {
+		return enable_derived_body(opt, packs, n_packs, pack_elems);
+	} catch (...) {
+		return -1;
+	}
+}
+
 float anni_adam_timed_derived_ms(const anni_adam *opt)
 {
 	return opt && opt->priv ? opt->priv->der_ms : 0.0f;
@@ -663,6 +693,7 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 	NormIn norm;
 	Flat f;
 	int np = 0;
+	int t;
 
 	if (!opt || !opt->priv)
 		return -1;
@@ -672,9 +703,9 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 		return -1;
 	pv = opt->priv;
 	st = compute_stream();
-	opt->t++;				/* lm_adam.c:533 */
-	c.bc1 = 1.0 - pow(opt->beta1, (double)opt->t);	/* lm_adam.c:571-572 */
-	c.bc2 = 1.0 - pow(opt->beta2, (double)opt->t);
+	t = opt->t + 1;				/* lm_adam.c:533; kept only when the step was launched */
+	c.bc1 = 1.0 - pow(opt->beta1, (double)t);	/* lm_adam.c:571-572 */
+	c.bc2 = 1.0 - pow(opt->beta2, (double)t);
 	if (c.bc1 <= 0.0 || c.bc2 <= 0.0)
 		return -1;			/* gpu_cuda.cu:8681-8682 */
 	c.rbc1 = 1.0 / c.bc1;
@@ -705,6 +736,7 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 		(void)hipEventRecord(ev[1], st);
 	if (launch_update(st, f, c, grad_scale, norm) != 0)
 		return -1;
+	opt->t = t;
 	if (ev)
 		(void)hipEventRecord(ev[2], st);
 	if (pv->fp8_twins) {
@@ -754,7 +786,7 @@ int anni_adam_sync_stats(anni_adam *opt)
 	return 0;
 }
 
-int anni_adam_time_steps(anni_adam *opt, int count, void *const *grads, int n_grads,
+static int time_steps_body(anni_adam *opt, int count, void *const *grads, int n_grads,
 	const double *lr, const double *grad_scale, float *ms_total, float *ms_sumsq,
 	float *ms_update)
 {
@@ -818,6 +850,18 @@ int anni_adam_time_steps(anni_adam *opt, int count, void *const *grads, int n_gr
 	for (size_t i = 0; i < ev.size(); i++)
 		(void)hipEventDestroy(ev[i]);
 	return rc;
+}
+
+int anni_adam_time_steps(anni_adam *opt, int count, void *const *grads, int n_grads,
+	const double *lr, const double *grad_scale, float *ms_total, float *ms_sumsq,
+	float *ms_update)
+{
+	try {
+		return time_steps_body(opt, count, grads, n_grads, lr, grad_scale, ms_total, ms_sumsq,
+		    ms_update);
+	} catch (...) {
+		return -1;
+	}
 }
 
 /* ---- optimizer block of a checkpoint (lang/lm_serialize.c:263-331,526-587) ----------- */
@@ -957,7 +1001,8 @@ static int read_all(int fd, void *buf, size_t n)
 int anni_adam_write_state(anni_adam *opt, int fd, int epoch, int step)
 {
 	int32_t head[5];
-	std::vector<float> buf;
+	float *buf;
+	int rc = 0;
 
 	if (!opt || !opt->priv || fd < 0 || opt->n > INT32_MAX)
 		return -1;
@@ -968,34 +1013,43 @@ int anni_adam_write_state(anni_adam *opt, int fd, int epoch, int step)
 	head[4] = (int32_t)opt->n;
 	if (write_all(fd, head, sizeof(head)) != 0)
 		return -1;
-	buf.resize((size_t)kCkptChunk * 2);
-	for (int64_t at = 0; at < opt->n; at += kCkptChunk) {
+	buf = (float *)malloc((size_t)kCkptChunk * 2 * sizeof(float));
+	if (!buf)
+		return -1;
+	for (int64_t at = 0; at < opt->n && rc == 0; at += kCkptChunk) {
 		const int64_t c = opt->n - at < kCkptChunk ? opt->n - at : kCkptChunk;
 
-		if (anni_adam_export_mv(opt, at, c, buf.data()) != 0
-		    || write_all(fd, buf.data(), (size_t)c * 2 * sizeof(float)) != 0)
-			return -1;
+		if (anni_adam_export_mv(opt, at, c, buf) != 0
+		    || write_all(fd, buf, (size_t)c * 2 * sizeof(float)) != 0)
+			rc = -1;
 	}
-	return 0;
+	free(buf);
+	return rc;
 }
 
 int anni_adam_read_state(anni_adam *opt, int fd, int *epoch, int *step)
 {
 	int32_t head[5];
-	std::vector<float> buf;
+	float *buf;
+	int rc = 0;
 
 	if (!opt || !opt->priv || fd < 0)
 		return -1;
 	if (read_all(fd, head, sizeof(head)) != 0 || head[0] != 1 || head[4] != opt->n)
 		return -1;		/* lm_serialize.c:546-562: has_adam == 1 and the same slot count */
-	buf.resize((size_t)kCkptChunk * 2);
-	for (int64_t at = 0; at < opt->n; at += kCkptChunk) {
+	buf = (float *)malloc((size_t)kCkptChunk * 2 * sizeof(float));
+	if (!buf)
+		return -1;
+	for (int64_t at = 0; at < opt->n && rc == 0; at += kCkptChunk) {
 		const int64_t c = opt->n - at < kCkptChunk ? opt->n - at : kCkptChunk;
 
-		if (read_all(fd, buf.data(), (size_t)c * 2 * sizeof(float)) != 0
-		    || anni_adam_import_mv(opt, at, c, buf.data()) != 0)
-			return -1;
+		if (read_all(fd, buf, (size_t)c * 2 * sizeof(float)) != 0
+		    || anni_adam_import_mv(opt, at, c, buf) != 0)
+			rc = -1;
 	}
+	free(buf);
+	if (rc != 0)
+		return -1;
 	opt->t = head[3];		/* so the learning-rate schedule continues (lm_serialize.c:564) */
 	if (epoch)
 		*epoch = head[1];

@@ -94,6 +94,80 @@ __global__ __launch_bounds__(kThreads) void copy16_kernel(void *dst, const void 
 		((u32x4 *)dst)[i] = ((const u32x4 *)src)[i];
 }
 
+/* ---- column sums in the host loop's order ----------------------------------------- */
+
+constexpr int kCsCols = 64;		/* columns per workgroup: one per lane of the summing wavefront */
+constexpr int kCsWaves = 8;
+constexpr int kCsRows = 16;		/* rows a wavefront fetches per round */
+constexpr int kCsRound = kCsWaves * kCsRows;
+
+/*
+** acc[c] = (...((acc[c] + t_0) + t_1) ... + t_{rows-1}) in float, t_r = x[r][c] (PROD: the float
+** product x[r][c] * y[r][c]), rows strictly in order: bit for bit what the reference's host
+** loops leave in a bias or LayerNorm gradient (lang/ffn.c:301-305,358-362,
+** lang/layernorm.c:368-372).  Float addition does not associate, so the chain of one column
+** cannot be split; what is spread out is everything else: a workgroup owns 64 columns, its
+** eight wavefronts keep 128 rows of loads in flight and park them in LDS, and while wavefront 0
+** walks one parked round in order the loads of the next round are already under way (two LDS
+** buffers, one barrier per round).  The chain costs a few cycles per row; the matrix streams
+** from HBM once, in 256-byte row segments.
+*/
+template <bool PROD>
+__global__ __launch_bounds__(kCsWaves * 64) void colsum_add_kernel(float *acc, const float *x,
+	const float *y, int64_t rows, int cols)
+{
+	__shared__ float park[2][kCsRound][kCsCols];
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const int64_t c = (int64_t)blockIdx.x * kCsCols + lane;
+	const bool live = c < cols;
+	const int64_t n_rounds = (rows + kCsRound - 1) / kCsRound;
+	float rx[kCsRows], ry[kCsRows];
+	float a = (wave == 0 && live) ? acc[c] : 0.0f;
+
+#pragma unroll
+	for (int i = 0; i < kCsRows; i++) {
+		const int64_t r = (int64_t)wave * kCsRows + i;
+		const bool in = live && r < rows;
+
+		rx[i] = in ? x[r * cols + c] : 0.0f;
+		ry[i] = (PROD && in) ? y[r * cols + c] : 1.0f;
+	}
+	for (int64_t round = 0; round < n_rounds; round++) {
+		float (*b)[kCsCols] = park[round & 1];
+
+#pragma unroll
+		for (int i = 0; i < kCsRows; i++)
+			b[wave * kCsRows + i][lane] = PROD ? rx[i] * ry[i] : rx[i];
+		__syncthreads();
+		if (round + 1 < n_rounds) {
+#pragma unroll
+			for (int i = 0; i < kCsRows; i++) {
+				const int64_t r = (round + 1) * kCsRound + (int64_t)wave * kCsRows + i;
+				const bool in = live && r < rows;
+
+				rx[i] = in ? x[r * cols + c] : 0.0f;
+				ry[i] = (PROD && in) ? y[r * cols + c] : 1.0f;
+			}
+		}
+		if (wave == 0) {
+			const int64_t left = rows - round * kCsRound;
+
+			if (left >= kCsRound) {
+#pragma unroll 16
+				for (int i = 0; i < kCsRound; i++)
+					a += b[i][lane];
+			} else {
+				/* rows past the end are never added: x + 0 is not x for x = -0 */
+				for (int i = 0; i < (int)left; i++)
+					a += b[i][lane];
+			}
+		}
+	}
+	if (wave == 0 && live)
+		acc[c] = a;
+}
+
 static int util_grid(int64_t items)
 {
 	int64_t g = (items + kThreads - 1) / kThreads;
@@ -136,6 +210,23 @@ int anni_copy_bytes(void *d_dst, const void *d_src, size_t nbytes)
 	hipLaunchKernelGGL(copy16_kernel, dim3(util_grid((int64_t)(nbytes / 16))), dim3(kThreads), 0,
 	    compute_stream(), d_dst, d_src, nbytes / 16);
 	return hip_ok(hipGetLastError(), "copy_bytes") ? 0 : -1;
+}
+
+int anni_colsum_add(float *d_acc, const float *d_x, const float *d_y, int64_t rows, int cols)
+{
+	const int64_t groups = ((int64_t)cols + kCsCols - 1) / kCsCols;
+
+	if (!d_acc || !d_x || rows < 0 || cols <= 0 || !device_ready())
+		return -1;
+	if (rows == 0)
+		return 0;
+	if (d_y)
+		hipLaunchKernelGGL((colsum_add_kernel<true>), dim3((unsigned)groups), dim3(kCsWaves * 64),
+		    0, compute_stream(), d_acc, d_x, d_y, rows, cols);
+	else
+		hipLaunchKernelGGL((colsum_add_kernel<false>), dim3((unsigned)groups),
+		    dim3(kCsWaves * 64), 0, compute_stream(), d_acc, d_x, d_y, rows, cols);
+	return hip_ok(hipGetLastError(), "colsum_add") ? 0 : -1;
 }
 
 int anni_fp8_quantize(void *d_q, float *d_scale, const float *d_src, int64_t n)

@@ -116,6 +116,7 @@ _PROTOS = {
     "anni_copy_bytes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "anni_f32_to_bf16": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64]),
     "anni_fp8_quantize": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]),
+    "anni_colsum_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]),
 }
 
 _lib = None

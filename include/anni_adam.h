@@ -220,6 +220,18 @@ int	anni_f32_to_bf16(void *d_dst, const float *d_src, int64_t n);
 ** d_scale[0] receives the scale; d_src is only read.
 */
 int	anni_fp8_quantize(void *d_q, float *d_scale, const float *d_src, int64_t n);
+/*
+** Bias / LayerNorm gradients straight into the gradient flat: d_acc[c] += column sums of the
+** row-major rows x cols matrix d_x (d_y given: of the element-wise float product d_x * d_y), added
+** one row after the other in float exactly as the reference's host loops do (lang/ffn.c:301-305,
+** 358-362: db += rows of dout / dh; lang/layernorm.c:368-372: dbeta += dy, dgamma += dy * x_hat),
+** so the result has the host path's bits and is the same on every run.  Stands where the
+** reference's device path keeps per-bias accumulators that it flushes to host vectors before the
+** optimizer gathers them again (gpu_mat_col_sum_add, num/gpu.h:195-199, gpu_cuda.cu:3131-3167):
+** with d_acc = (float *)opt->d_grad + anni_adam_tensor_offset(opt, i) nothing leaves the device.
+** rows == 0 leaves d_acc alone.
+*/
+int	anni_colsum_add(float *d_acc, const float *d_x, const float *d_y, int64_t rows, int cols);
 
 #ifdef __cplusplus
 }

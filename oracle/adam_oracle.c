@@ -487,3 +487,24 @@ void oracle_adam_step_slots(oracle_slot *slots, int64_t n, int t, double beta1,
 		*slots[i].grad = 0.0f;
 	}
 }
+
+/*
+** Column sums in the order of the reference's host loops (lang/ffn.c:301-305,358-362:
+** db[j] += x[t * cols + j]; lang/layernorm.c:368-372: dbeta[j] += dy, dgamma[j] += dy * x_hat),
+** rows outermost, everything in float: acc[j] = (acc[j] + t_0) + t_1 ... with t the element or the
+** float product of the two elements.
+*/
+void oracle_colsum_add(float *acc, const float *x, const float *y, int64_t rows, int cols)
+{
+	int64_t t;
+	int j;
+
+	for (t = 0; t < rows; t++) {
+		for (j = 0; j < cols; j++) {
+			if (y)
+				acc[j] += x[t * cols + j] * y[t * cols + j];
+			else
+				acc[j] += x[t * cols + j];
+		}
+	}
+}

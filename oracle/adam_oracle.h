@@ -16,11 +16,14 @@
 **   oracle_bf16_rne                num/gpu_cuda.cu:8578,1505 (__float2bfloat16 = RNE)
 **   oracle_fp8_scale_from_amax     num/gpu_cuda.cu:927-938 (amax_to_scale_kernel)
 **   oracle_fp8_quantize            num/gpu_cuda.cu:826-851 (x * (1/scale), satfinite E4M3)
+**   oracle_colsum_add              lang/ffn.c:301-305,358-362, lang/layernorm.c:368-372
+**                                  (bias / LayerNorm gradients as serial float column sums)
 **
 ** Pinned by: the reference's compiled lm_adam_step_scaled (oracle/_ref, bit for
 ** bit on p/m/v), the reference's own LR known answers (tests/test_ann.c:866-879),
 ** closed forms (t=1, constant gradient, zero gradient), and brute-force
-** long-double sums.  PARITY UNPINNED by the reference (no implementation exists
+** long-double sums; oracle_colsum_add by the reference's compiled layernorm_backward
+** (dgamma / dbeta, bit for bit) and by inputs whose sum depends on the order.  PARITY UNPINNED by the reference (no implementation exists
 ** there, the oracle defines them): bf16-stored m/v, bf16 gradients, fp8-E4M3
 ** gradients with a per-tensor scale, weight decay on selected tensors only, and
 ** the non-finite skip on the CPU path.
@@ -116,6 +119,9 @@ typedef struct oracle_slot {
 void	oracle_adam_step_slots(oracle_slot *slots, int64_t n, int t, double beta1,
 		double beta2, double eps, double weight_decay, double grad_clip,
 		double lr, double grad_scale);
+
+/* acc[j] += column sums of x (y != NULL: of x * y), rows x cols row-major, the host loops' order. */
+void	oracle_colsum_add(float *acc, const float *x, const float *y, int64_t rows, int cols);
 
 int	oracle_max_threads(void);
 

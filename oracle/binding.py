@@ -169,6 +169,29 @@ def fp8_decode_table():
     return np.array([lib().oracle_fp8_decode(q) for q in range(256)], dtype=np.float32)
 
 
+def colsum_add(acc, x, y=None):
+    """acc[j] += column sums of the 2-D float32 array x (of x * y), in place, host-loop order."""
+    assert acc.dtype == np.float32 and x.dtype == np.float32 and x.flags.c_contiguous
+    rows, cols = x.shape
+    assert acc.size == cols and (y is None or (y.shape == x.shape and y.dtype == np.float32))
+    L = lib()
+    L.oracle_colsum_add.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
+    L.oracle_colsum_add.restype = None
+    L.oracle_colsum_add(_ptr(acc), _ptr(x), _ptr(y) if y is not None else None, rows, cols)
+    return acc
+
+
+def ref_ln_backward_grads(dy, x_hat, dgamma, dbeta):
+    """The compiled reference's layernorm_backward: accumulates into dgamma / dbeta in place."""
+    R = ref()
+    R.ref_ln_backward_grads.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+    R.ref_ln_backward_grads.restype = C.c_int
+    assert dy.dtype == np.float32 and dy.shape == x_hat.shape and dy.flags.c_contiguous
+    d = R.ref_ln_backward_grads(_ptr(dy), _ptr(x_hat), dy.shape[0], _ptr(dgamma), _ptr(dbeta))
+    if d != dy.shape[1]:
+        raise RuntimeError("ref_ln_backward_grads: %d" % d)
+
+
 def fp8_quantize(x):
     """float32 tensor -> (uint8 codes, float scale) by the per-tensor amax convention."""
     x = np.ascontiguousarray(x, dtype=np.float32)

@@ -14,6 +14,7 @@
 #include "lm_adam.h"
 #include "lm_serialize.h"
 #include "lm_train.h"
+#include "layernorm.h"
 
 typedef struct ref_adam {
 	lm_adam	opt;
@@ -277,6 +278,44 @@ void ref_model_free(ref_model *r)
 	lm_adam_free(&r->opt);
 	lm_free(&r->model);
 	free(r);
+}
+
+/*
+** dgamma / dbeta as the reference's host layernorm_backward accumulates them
+** (lang/layernorm.c:312-376; model width LM_D_MODEL is a compile-time constant): both start
+** from the given values, dy and x_hat are T x LM_D_MODEL row-major.  Returns LM_D_MODEL, -1 on failure.
+*/
+int ref_ln_backward_grads(const float *dy, const float *x_hat, int T, float *dgamma, float *dbeta)
+{
+	layernorm *ln = layernorm_create();
+	ln_cache *c = ln_cache_create(T);
+	mat *mdy = mat_create(T, LM_D_MODEL);
+	mat *mdx = mat_create(T, LM_D_MODEL);
+	int rc = -1;
+	int i;
+
+	if (c && !c->x_hat)		/* not stored when the device recomputes it (layernorm.c:116-121) */
+		c->x_hat = mat_create(T, LM_D_MODEL);
+	if (ln && c && mdy && mdx && c->x_hat && c->inv_std) {
+		memcpy(mdy->data, dy, (size_t)T * LM_D_MODEL * sizeof(float));
+		memcpy(c->x_hat->data, x_hat, (size_t)T * LM_D_MODEL * sizeof(float));
+		for (i = 0; i < T; i++)
+			c->inv_std->data[i] = 1.0f;
+		c->T = T;
+		c->x_src = NULL;
+		memcpy(ln->dgamma->data, dgamma, LM_D_MODEL * sizeof(float));
+		memcpy(ln->dbeta->data, dbeta, LM_D_MODEL * sizeof(float));
+		if (layernorm_backward(mdx, mdy, ln, c) == 0) {
+			memcpy(dgamma, ln->dgamma->data, LM_D_MODEL * sizeof(float));
+			memcpy(dbeta, ln->dbeta->data, LM_D_MODEL * sizeof(float));
+			rc = LM_D_MODEL;
+		}
+	}
+	mat_free(&mdy);
+	mat_free(&mdx);
+	ln_cache_free(&c);
+	layernorm_free(&ln);
+	return rc;
 }
 
 double ref_step_lr(double base_lr, int step, int warmup, int decay_steps,

@@ -3,12 +3,15 @@
 Run in a container that holds the reference tree (oracle/Makefile builds
 oracle/_ref/libanni_ref.so from the reference's sources where they lie):
 
-    python tests/golden/make_golden.py
+    python tests/golden/make_golden.py            # everything
+    python tests/golden/make_golden.py ln_colsum  # only the named fixtures
 
 Each fixture holds seeded inputs (p0, one gradient per step, hyper-parameters,
 the per-step lr and grad_scale) and what the reference's lm_adam_step_scaled host
 path (lang/lm_adam.c:559-606) produced after every step (p, m, v).  The learning
 rates come from the reference's lm_train_step_lr (lang/lm_train.c:98-124).
+ln_colsum holds the bias / LayerNorm gradient sums: dgamma and dbeta as the reference's
+host layernorm_backward (lang/layernorm.c:312-376) accumulates them over seeded dy and x_hat.
 Fixtures are data only; the GPU box re-checks the oracle and the HIP path
 against them without the reference being present.
 """
@@ -44,11 +47,37 @@ CASES = {
 }
 
 
-def main():
+def ln_colsum():
+    """Inputs whose float column sums depend on the order of the additions: magnitudes spread
+    over eight decades, exact cancellations, signed zeros, accumulators that do not start at 0."""
+    rng = np.random.default_rng(21)
+    T, d = 19, 1024
+    dy = (rng.standard_normal((T, d)) * 10.0 ** rng.integers(-4, 4, (T, d))).astype(np.float32)
+    xh = rng.standard_normal((T, d)).astype(np.float32)
+    dy[0, :8] = 1e8
+    dy[1, :8] = 1.0
+    dy[2, :8] = -1e8                       # (1e8 + 1) - 1e8 = 0 in float, 1 in any other order
+    dy[:, 8] = -0.0                        # a column of -0: the sum stays -0 from a -0 start
+    xh[:, 9] = 0.0
+    dgamma0 = (rng.standard_normal(d) * 1e-2).astype(np.float32)
+    dbeta0 = (rng.standard_normal(d) * 1e-2).astype(np.float32)
+    dbeta0[8] = -0.0
+    dgamma, dbeta = dgamma0.copy(), dbeta0.copy()
+    ob.ref_ln_backward_grads(dy, xh, dgamma, dbeta)
+    np.savez_compressed(os.path.join(HERE, "ln_colsum.npz"), dy=dy, x_hat=xh, dgamma0=dgamma0,
+                        dbeta0=dbeta0, dgamma=dgamma, dbeta=dbeta)
+    print("wrote ln_colsum", T, d)
+
+
+def main(only=()):
     if not ob.ref_available():
         raise SystemExit("oracle/_ref/libanni_ref.so is missing: run `make -C oracle` "
                          "where the reference tree is present")
+    if not only or "ln_colsum" in only:
+        ln_colsum()
     for name, c in CASES.items():
+        if only and name not in only:
+            continue
         rng = np.random.default_rng(c["seed"])
         n = c["n"]
         p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
@@ -85,6 +114,8 @@ def main():
             wd=np.float64(c["wd"]), clip=np.float64(c["clip"]),
             p=np.stack(P), m=np.stack(M), v=np.stack(V))
         print("wrote", name, n)
+    if only and "lr_table" not in only:
+        return
     # learning-rate table straight from lm_train_step_lr
     steps = np.array([0, 1, 9, 50, 98, 99, 100, 101, 350, 600, 1099, 1100, 1101, 5000], np.int32)
     rows = []
@@ -101,4 +132,4 @@ def main():
 
 
 if __name__ == "__main__":
-    main()
+    main(tuple(sys.argv[1:]))

@@ -361,3 +361,50 @@ def test_storage_modes_round_where_documented(oracle):
     g_d = (oracle.fp8_decode_table()[q] * s).astype(np.float32)
     oracle.Oracle(n, beta2=0.95).step(p_d, g_d, m_d, v_d, 3e-4)
     assert same_bits(p_c, p_d) and same_bits(m_c, m_d) and same_bits(v_c, v_d) and not qq.any()
+
+
+# ---- bias / LayerNorm gradient column sums ---------------------------------------------------
+
+def test_colsum_matches_golden_of_the_reference(oracle):
+    """dgamma / dbeta written by the reference's compiled host layernorm_backward."""
+    G = load_golden("ln_colsum")
+    dbeta = oracle.colsum_add(G["dbeta0"].copy(), G["dy"])
+    dgamma = oracle.colsum_add(G["dgamma0"].copy(), G["dy"], G["x_hat"])
+    assert same_bits(dbeta, G["dbeta"]) and same_bits(dgamma, G["dgamma"])
+    assert np.signbit(G["dbeta"][8]) and G["dbeta"][8] == 0.0        # -0 + (-0) ... stays -0
+
+
+def test_colsum_equals_compiled_reference(oracle):
+    if not oracle.ref_available():
+        pytest.skip("compiled reference absent")
+    rng = np.random.default_rng(8)
+    for T in (1, 2, 63, 130):
+        dy = (rng.standard_normal((T, 1024)) * 10.0 ** rng.integers(-3, 3, (T, 1024))).astype(np.float32)
+        xh = rng.standard_normal((T, 1024)).astype(np.float32)
+        g0 = rng.standard_normal(1024).astype(np.float32)
+        b0 = rng.standard_normal(1024).astype(np.float32)
+        g, b = g0.copy(), b0.copy()
+        oracle.ref_ln_backward_grads(dy, xh, g, b)
+        assert same_bits(oracle.colsum_add(b0.copy(), dy), b)
+        assert same_bits(oracle.colsum_add(g0.copy(), dy, xh), g)
+
+
+def test_colsum_order_and_rounding_known_answers(oracle):
+    """Cases where another order, a wider accumulator or a fused multiply-add gives another
+    float: the answers below follow from IEEE single arithmetic alone."""
+    x = np.array([[1e8], [1.0], [-1e8], [1.0]], np.float32)
+    assert oracle.colsum_add(np.zeros(1, np.float32), x)[0] == 1.0      # ((0+1e8)+1)-1e8 = 0, +1
+    assert oracle.colsum_add(np.ones(1, np.float32), x[::-1].copy())[0] == 0.0   # (((1+1)-1e8)+1)+1e8
+    # 2^24 + 1 + 1 = 2^24 serially (each 1 is lost); a double accumulator would give 2^24 + 2
+    x = np.array([[1.0], [1.0]], np.float32)
+    assert oracle.colsum_add(np.array([2.0 ** 24], np.float32), x)[0] == 2.0 ** 24
+    # the product is rounded to float before it is added: a = 1 + 2^-12, a*a = 1 + 2^-11 + 2^-24
+    # rounds to 1 + 2^-11; adding -(1 + 2^-11) gives exactly 0, a fused multiply-add 2^-24
+    a = np.float32(1.0 + 2.0 ** -12)
+    x = np.array([[a]], np.float32)
+    acc = np.array([-(1.0 + 2.0 ** -11)], np.float32)
+    assert oracle.colsum_add(acc, x, x.copy())[0] == 0.0
+    # zero rows: nothing is added, a -0 accumulator keeps its sign
+    acc = np.array([-0.0, 3.0], np.float32)
+    out = oracle.colsum_add(acc, np.zeros((0, 2), np.float32))
+    assert np.signbit(out[0]) and out[1] == 3.0
