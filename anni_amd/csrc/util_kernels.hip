@@ -96,76 +96,161 @@ __global__ __launch_bounds__(kThreads) void copy16_kernel(void *dst, const void 
 
 /* ---- column sums in the host loop's order ----------------------------------------- */
 
-constexpr int kCsCols = 64;		/* columns per workgroup: one per lane of the summing wavefront */
+constexpr int kCsCols = 64;		/* columns per workgroup: one per lane */
 constexpr int kCsWaves = 8;
-constexpr int kCsRows = 16;		/* rows a wavefront fetches per round */
-constexpr int kCsRound = kCsWaves * kCsRows;
+/*
+** Rows per chunk = what one wavefront holds in registers.  (With two matrices a chunk is 128
+** loads, more than the 63 a wavefront can have outstanding, so that variant waits inside its
+** fetches and runs at about half the rate; 32-row chunks were measured slower still, the
+** hand-over between wavefronts then costs more than the waits.)
+*/
+template <bool PROD> struct CsRows { static constexpr int n = 64; };
+
+/*
+** Rows FIRST .. FIRST + COUNT - 1 of a chunk of the lane's column into registers, as raw buffer loads: the
+** descriptor (scalar registers) starts at the chunk's first row and ends with the matrix, the
+** row offset is a scalar, the lane supplies only its constant column offset -- no vector
+** arithmetic per load, and a row past the end reads as 0 without touching memory (those
+** registers are never added).  A select on a loaded value instead would make the wavefront
+** wait for the load on the spot.
+*/
+template <bool PROD, int FIRST, int COUNT>
+__device__ __forceinline__ void colsum_fetch(float (&rx)[CsRows<PROD>::n], float (&ry)[CsRows<PROD>::n],
+	const float *x, const float *y, int64_t chunk, int64_t rows, int cols, uint32_t col_bytes)
+{
+	constexpr int kCsRows = CsRows<PROD>::n;
+	const int64_t r0 = chunk * kCsRows;
+
+	if (r0 >= rows)
+		return;
+	const uint64_t left = (uint64_t)(rows - r0) * (uint64_t)cols * sizeof(float);
+	const uint32_t span = left < 0xffffffffull ? (uint32_t)left : 0xffffffffu;
+	const __amdgpu_buffer_rsrc_t bx = __builtin_amdgcn_make_buffer_rsrc(
+	    (void *)(x + r0 * cols), 0, (int)span, 0x00020000);
+	const __amdgpu_buffer_rsrc_t by = __builtin_amdgcn_make_buffer_rsrc(
+	    (void *)((PROD ? y : x) + r0 * cols), 0, (int)span, 0x00020000);
+	const uint32_t pitch = (uint32_t)cols * (uint32_t)sizeof(float);
+
+#pragma unroll
+	for (int i = FIRST; i < FIRST + COUNT; i++) {
+		rx[i] = __builtin_bit_cast(float,
+		    __builtin_amdgcn_raw_buffer_load_b32(bx, (int)col_bytes, (int)(i * pitch), 0));
+		if (PROD)
+			ry[i] = __builtin_bit_cast(float,
+			    __builtin_amdgcn_raw_buffer_load_b32(by, (int)col_bytes, (int)(i * pitch), 0));
+	}
+}
 
 /*
 ** acc[c] = (...((acc[c] + t_0) + t_1) ... + t_{rows-1}) in float, t_r = x[r][c] (PROD: the float
 ** product x[r][c] * y[r][c]), rows strictly in order: bit for bit what the reference's host
 ** loops leave in a bias or LayerNorm gradient (lang/ffn.c:301-305,358-362,
 ** lang/layernorm.c:368-372).  Float addition does not associate, so the chain of one column
-** cannot be split; what is spread out is everything else: a workgroup owns 64 columns, its
-** eight wavefronts keep 128 rows of loads in flight and park them in LDS, and while wavefront 0
-** walks one parked round in order the loads of the next round are already under way (two LDS
-** buffers, one barrier per round).  The chain costs a few cycles per row; the matrix streams
-** from HBM once, in 256-byte row segments.
+** cannot be split; what is spread out is the memory traffic.  A workgroup owns 64 columns, one
+** per lane.  Its eight wavefronts take chunks of 64 rows in turn: a wavefront holds its chunk
+** in registers (loaded several turns earlier), picks the running sums up from LDS, adds its
+** rows in order and hands the sums on; during the four following turns it fetches the chunk of
+** its next turn.  So ~100 KiB per workgroup are in flight while the chain runs at register speed,
+** or at the HBM rate where the matrix is wide.  One barrier per chunk; no wavefront ever waits
+** for a later one.
 */
 template <bool PROD>
 __global__ __launch_bounds__(kCsWaves * 64) void colsum_add_kernel(float *acc, const float *x,
 	const float *y, int64_t rows, int cols)
 {
-	__shared__ float park[2][kCsRound][kCsCols];
+	constexpr int kCsRows = CsRows<PROD>::n;
+	__shared__ float carry[kCsCols];
 	const int lane = threadIdx.x & 63;
-	const int wave = threadIdx.x >> 6;
-	const int64_t c = (int64_t)blockIdx.x * kCsCols + lane;
-	const bool live = c < cols;
-	const int64_t n_rounds = (rows + kCsRound - 1) / kCsRound;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const int64_t c_own = (int64_t)blockIdx.x * kCsCols + lane;
+	const bool live = c_own < cols;
+	const uint32_t c = (uint32_t)(live ? c_own : cols - 1);
+	const uint32_t col_bytes = c * (uint32_t)sizeof(float);
+	const int64_t n_chunks = (rows + kCsRows - 1) / kCsRows;
+	int64_t done = 0;		/* chunks added so far = barriers passed, the same in every wavefront */
 	float rx[kCsRows], ry[kCsRows];
-	float a = (wave == 0 && live) ? acc[c] : 0.0f;
 
-#pragma unroll
-	for (int i = 0; i < kCsRows; i++) {
-		const int64_t r = (int64_t)wave * kCsRows + i;
-		const bool in = live && r < rows;
-
-		rx[i] = in ? x[r * cols + c] : 0.0f;
-		ry[i] = (PROD && in) ? y[r * cols + c] : 1.0f;
-	}
-	for (int64_t round = 0; round < n_rounds; round++) {
-		float (*b)[kCsCols] = park[round & 1];
-
+	if (wave == 0)
+		carry[lane] = acc[c];
+	colsum_fetch<PROD, 0, kCsRows>(rx, ry, x, y, wave, rows, cols, col_bytes);
+	if (PROD) {
+		/* products are rounded to float before they are added: no fused multiply-add */
 #pragma unroll
 		for (int i = 0; i < kCsRows; i++)
-			b[wave * kCsRows + i][lane] = PROD ? rx[i] * ry[i] : rx[i];
+			rx[i] = rx[i] * ry[i];
+	}
+	__syncthreads();
+	/*
+	** Every wavefront runs the same cycle of eight chunks -- own turn, four chunks during each
+	** of which it fetches a quarter of its next chunk, two idle chunks, multiply -- shifted by its
+	** index, with one barrier per chunk.  (One loop with the phase as a run-time value made the
+	** compiler copy the row registers at the loop end, which waits for every load in flight.)
+	*/
+	for (int k = 0; k < wave && done < n_chunks; k++) {
 		__syncthreads();
-		if (round + 1 < n_rounds) {
+		done++;
+	}
+	while (done < n_chunks) {
+		{
+			const int64_t left = rows - done * kCsRows;
+			float a = carry[lane];
+
+			if (left >= kCsRows) {
 #pragma unroll
-			for (int i = 0; i < kCsRows; i++) {
-				const int64_t r = (round + 1) * kCsRound + (int64_t)wave * kCsRows + i;
-				const bool in = live && r < rows;
-
-				rx[i] = in ? x[r * cols + c] : 0.0f;
-				ry[i] = (PROD && in) ? y[r * cols + c] : 1.0f;
-			}
-		}
-		if (wave == 0) {
-			const int64_t left = rows - round * kCsRound;
-
-			if (left >= kCsRound) {
-#pragma unroll 16
-				for (int i = 0; i < kCsRound; i++)
-					a += b[i][lane];
+				for (int i = 0; i < kCsRows; i++)
+					a += rx[i];
 			} else {
 				/* rows past the end are never added: x + 0 is not x for x = -0 */
-				for (int i = 0; i < (int)left; i++)
-					a += b[i][lane];
+#pragma unroll
+				for (int i = 0; i < kCsRows; i++)
+					if (i < left)
+						a += rx[i];
 			}
+			carry[lane] = a;
 		}
+		__syncthreads();
+		if (++done >= n_chunks)
+			break;
+		/*
+		** Not inside the own turn, and a quarter at a time: issuing the loads of a whole chunk takes
+		** as long as the chain of one, and would hold up the barrier the next chain waits on.
+		*/
+		colsum_fetch<PROD, 0, kCsRows / 4>(rx, ry, x, y, done - 1 + kCsWaves, rows, cols, col_bytes);
+		__syncthreads();
+		if (++done >= n_chunks)
+			break;
+		colsum_fetch<PROD, kCsRows / 4, kCsRows / 4>(rx, ry, x, y, done - 2 + kCsWaves, rows, cols,
+		    col_bytes);
+		__syncthreads();
+		if (++done >= n_chunks)
+			break;
+		colsum_fetch<PROD, kCsRows / 2, kCsRows / 4>(rx, ry, x, y, done - 3 + kCsWaves, rows, cols,
+		    col_bytes);
+		__syncthreads();
+		if (++done >= n_chunks)
+			break;
+		colsum_fetch<PROD, 3 * kCsRows / 4, kCsRows / 4>(rx, ry, x, y, done - 4 + kCsWaves, rows,
+		    cols, col_bytes);
+		__syncthreads();
+		if (++done >= n_chunks)
+			break;
+#pragma unroll 1
+		for (int k = 5; k < kCsWaves - 1 && done < n_chunks; k++) {
+			__syncthreads();
+			done++;
+		}
+		if (done >= n_chunks)
+			break;
+		if (PROD) {
+#pragma unroll
+			for (int i = 0; i < kCsRows; i++)
+				rx[i] = rx[i] * ry[i];
+		}
+		__syncthreads();
+		done++;
 	}
 	if (wave == 0 && live)
-		acc[c] = a;
+		acc[c] = carry[lane];
 }
 
 static int util_grid(int64_t items)

@@ -194,6 +194,34 @@ def reference_caller_leg(L):
             "GBps_algorithmic": round(n * 38 / ms / 1e6, 1)}
 
 
+def colsum_leg(L, rows, shapes=((6272, False), (1536, False), (1536, True))):
+    """anni_colsum_add at the 555M model's shapes: db1 (rows x 6272), db2 / dbeta (rows x 1536),
+    dgamma (rows x 1536, product of two matrices); 20 launches each, wall clock around them."""
+    from anni_amd.lm_adam import DeviceBuffer
+    out = []
+    for cols, prod in shapes:
+        n = rows * cols
+        x, y, acc = DeviceBuffer(n * 4), DeviceBuffer(n * 4), DeviceBuffer(cols * 4)
+        assert L.anni_fill_normal_f32(x.ptr, n, 5, 1, 0.0, 1e-2) == 0
+        assert L.anni_fill_normal_f32(y.ptr, n, 5, 2, 0.0, 1.0) == 0
+        assert L.gpu_memset(acc.ptr, 0, cols * 4) == 0
+        for _ in range(3):
+            assert L.anni_colsum_add(acc.ptr, x.ptr, y.ptr if prod else None, rows, cols) == 0
+        L.gpu_device_sync()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            assert L.anni_colsum_add(acc.ptr, x.ptr, y.ptr if prod else None, rows, cols) == 0
+        L.gpu_device_sync()
+        ms = (time.perf_counter() - t0) * 1e3 / 20
+        nbytes = n * 4 * (2 if prod else 1)
+        out.append({"rows": rows, "cols": cols, "product": prod, "ms": round(ms, 4),
+                    "bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1),
+                    "ns_per_row": round(ms * 1e6 / rows, 2)})
+        for b in (x, y, acc):
+            b.free()
+    return out
+
+
 def copy_calibration(L, nbytes):
     """Ten launches of the plain copy kernel: each reads nbytes and writes nbytes exactly."""
     from anni_amd.lm_adam import DeviceBuffer
@@ -222,6 +250,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="only run the plain copy kernel over BYTES ten times (counter calibration)")
+    ap.add_argument("--colsum", type=int, default=0, metavar="ROWS",
+                    help="only time the bias / LayerNorm gradient column sums over ROWS token rows")
     ap.add_argument("--reference-caller-only", action="store_true",
                     help="only time the unchanged reference caller on this backend (one JSON line)")
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds for the CPU legs")
@@ -250,6 +280,9 @@ def main():
         env = bench_row.probe_env(L, os.path.dirname(os.path.abspath(__file__)))
     if a.copy_calibration:
         copy_calibration(L, a.copy_calibration)
+        return
+    if a.colsum:
+        print(json.dumps({"colsum_add": colsum_leg(L, a.colsum)}))
         return
     if a.reference_caller_only:
         print(json.dumps(reference_caller_leg(L)))
