@@ -301,7 +301,8 @@ int anni_colsum_add(float *d_acc, const float *d_x, const float *d_y, int64_t ro
 {
 	const int64_t groups = ((int64_t)cols + kCsCols - 1) / kCsCols;
 
-	if (!d_acc || !d_x || rows < 0 || cols <= 0 || !device_ready())
+	/* 63 row pitches must fit the 32-bit scalar offset of a buffer load */
+	if (!d_acc || !d_x || rows < 0 || cols <= 0 || cols > (1 << 24) || !device_ready())
 		return -1;
 	if (rows == 0)
 		return 0;

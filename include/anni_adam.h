@@ -229,7 +229,7 @@ int	anni_fp8_quantize(void *d_q, float *d_scale, const float *d_src, int64_t n);
 ** reference's device path keeps per-bias accumulators that it flushes to host vectors before the
 ** optimizer gathers them again (gpu_mat_col_sum_add, num/gpu.h:195-199, gpu_cuda.cu:3131-3167):
 ** with d_acc = (float *)opt->d_grad + anni_adam_tensor_offset(opt, i) nothing leaves the device.
-** rows == 0 leaves d_acc alone.
+** rows == 0 leaves d_acc alone; cols up to 2^24.
 */
 int	anni_colsum_add(float *d_acc, const float *d_x, const float *d_y, int64_t rows, int cols);
 

@@ -131,5 +131,6 @@ def test_argument_checks(gpu):
     assert gpu.anni_colsum_add(d.ptr, None, None, 4, 4) == -1
     assert gpu.anni_colsum_add(d.ptr, d.ptr, None, -1, 4) == -1
     assert gpu.anni_colsum_add(d.ptr, d.ptr, None, 4, 0) == -1
+    assert gpu.anni_colsum_add(d.ptr, d.ptr, None, 4, (1 << 24) + 1) == -1
     assert gpu.anni_colsum_add(d.ptr, d.ptr, None, 0, 4) == 0
     d.free()
