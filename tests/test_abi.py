@@ -134,3 +134,26 @@ def test_layout_parameter_counts():
     assert len(layout.tensors("555m", "reference")) == 2 + 12 * 14
     mats = [t for t in layout.tensors("555m") if t[2]]
     assert all(n >= 1536 * 1536 for _nm, n, _f in mats)
+
+
+def test_c99_caller_with_the_reference_flags(tmp_path):
+    """include/*.h are plain C99 under the reference's own compiler flags (Makefile:21), and a C
+    program links against the library and gets the schedule's known answers
+    (tests/test_ann.c:866-879: 0.01 at step 0 of a 100-step warmup, 1.0 at step 99, 0.5 half way
+    down the cosine, 0 at its end)."""
+    import shutil
+    import subprocess
+    from anni_amd import lib
+    if not shutil.which("gcc"):
+        pytest.skip("no gcc")
+    exe = str(tmp_path / "abi_probe")
+    libdir = os.path.dirname(lib.SO_PATH)
+    subprocess.check_call(["gcc", "-W", "-Wall", "-Werror", "-ansi", "-pedantic", "-std=c99", "-O2",
+                           "-I", os.path.join(ROOT, "include"),
+                           os.path.join(ROOT, "tests", "c", "abi_probe.c"), "-o", exe,
+                           "-L", libdir, "-lanni_gpu_hip", "-Wl,-rpath," + libdir, "-lm"])
+    out = subprocess.check_output([exe], timeout=120).decode().splitlines()
+    lr = [float(x) for x in out[0].split()[1:]]
+    assert lr[0] == 0.01 and lr[1] == 1.0 and abs(lr[2] - 0.5) < 1e-15 and abs(lr[3]) < 1e-15
+    assert out[1].startswith("backend hip-gfx950 available ")
+    assert out[2].startswith("create declined") or out[2].startswith("create ok n 4160 t 1 norm 0")
