@@ -15,6 +15,7 @@
 #include <vector>
 #include "adam_kernels.h"
 #include "anni_adam.h"
+#include "anni_gpu.h"
 #include "backend_state.h"
 
 using namespace anni;
@@ -750,6 +751,11 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 	}
 	if (ev)
 		(void)hipEventRecord(ev[3], st);
+	/*
+	** The weights moved: consumers that cache derived copies keyed on the weight epoch rebuild
+	** them (lm_adam.c:541-547 does this after every device step, a skipped one included).
+	*/
+	gpu_half_wt_invalidate(nullptr);
 	return 0;
 }
 

@@ -158,9 +158,13 @@ def test_golden_vectors_through_arena(gpu, oracle):
 def test_lr_nonpositive_is_a_noop(gpu):
     opt = make(gpu, [(100, 3)])
     opt.upload("grad", np.ones(100, np.float32))
+    e0 = gpu.gpu_param_epoch()
     assert opt.step_scaled(0.0) == 1 and opt.t == 0          # lm_adam.c:531-532
     assert opt.step_scaled(-1.0) == 1 and opt.t == 0
     assert opt.download("grad").all() and not opt.download("param").any()
+    assert gpu.gpu_param_epoch() == e0                        # nothing moved
+    assert opt.step_scaled(1e-3) == 0 and opt.t == 1
+    assert gpu.gpu_param_epoch() == e0 + 1                    # lm_adam.c:547: the weight epoch moves
     opt.free()
 
 
