@@ -154,15 +154,40 @@ __device__ __forceinline__ void colsum_fetch(float (&rx)[CsRows<PROD>::n], float
 ** or at the HBM rate where the matrix is wide.  One barrier per chunk; no wavefront ever waits
 ** for a later one.
 */
+constexpr int kCsMaxJobs = 16;
+
+/* One column sum of a launch; the jobs of a launch travel by value in the kernel arguments. */
+struct CsJob {
+	float		*acc;
+	const float	*x;
+	const float	*y;
+	int64_t		rows;
+	int		cols;
+	int		first_group;	/* workgroups [first_group, next job's first_group) work on this job */
+};
+
+struct CsJobs {
+	int	n;
+	CsJob	job[kCsMaxJobs];
+};
+
 template <bool PROD>
-__global__ __launch_bounds__(kCsWaves * 64) void colsum_add_kernel(float *acc, const float *x,
-	const float *y, int64_t rows, int cols)
+__global__ __launch_bounds__(kCsWaves * 64) void colsum_add_kernel(CsJobs jobs)
 {
 	constexpr int kCsRows = CsRows<PROD>::n;
 	__shared__ float carry[kCsCols];
 	const int lane = threadIdx.x & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-	const int64_t c_own = (int64_t)blockIdx.x * kCsCols + lane;
+	int k = 0;
+
+	while (k + 1 < jobs.n && (int)blockIdx.x >= jobs.job[k + 1].first_group)
+		k++;
+	float *const acc = jobs.job[k].acc;
+	const float *const x = jobs.job[k].x;
+	const float *const y = jobs.job[k].y;
+	const int64_t rows = jobs.job[k].rows;
+	const int cols = jobs.job[k].cols;
+	const int64_t c_own = (int64_t)((int)blockIdx.x - jobs.job[k].first_group) * kCsCols + lane;
 	const bool live = c_own < cols;
 	const uint32_t c = (uint32_t)(live ? c_own : cols - 1);
 	const uint32_t col_bytes = c * (uint32_t)sizeof(float);
@@ -297,22 +322,53 @@ int anni_copy_bytes(void *d_dst, const void *d_src, size_t nbytes)
 	return hip_ok(hipGetLastError(), "copy_bytes") ? 0 : -1;
 }
 
+int anni_colsum_add_batch(const anni_colsum *jobs, int n_jobs)
+{
+	CsJobs plain, prod;
+	int groups[2] = { 0, 0 };
+
+	if (!jobs || n_jobs <= 0 || n_jobs > kCsMaxJobs || !device_ready())
+		return -1;
+	plain.n = 0;
+	prod.n = 0;
+	for (int i = 0; i < n_jobs; i++) {
+		const anni_colsum &j = jobs[i];
+
+		/* 63 row pitches must fit the 32-bit scalar offset of a buffer load */
+		if (!j.d_acc || !j.d_x || j.rows < 0 || j.cols <= 0 || j.cols > (1 << 24))
+			return -1;
+		if (j.rows == 0)
+			continue;
+		CsJobs &dst = j.d_y ? prod : plain;
+		CsJob &c = dst.job[dst.n++];
+
+		c.acc = j.d_acc;
+		c.x = j.d_x;
+		c.y = j.d_y;
+		c.rows = j.rows;
+		c.cols = j.cols;
+		c.first_group = groups[j.d_y ? 1 : 0];
+		groups[j.d_y ? 1 : 0] += (j.cols + kCsCols - 1) / kCsCols;
+	}
+	if (plain.n)
+		hipLaunchKernelGGL((colsum_add_kernel<false>), dim3((unsigned)groups[0]),
+		    dim3(kCsWaves * 64), 0, compute_stream(), plain);
+	if (prod.n)
+		hipLaunchKernelGGL((colsum_add_kernel<true>), dim3((unsigned)groups[1]),
+		    dim3(kCsWaves * 64), 0, compute_stream(), prod);
+	return hip_ok(hipGetLastError(), "colsum_add") ? 0 : -1;
+}
+
 int anni_colsum_add(float *d_acc, const float *d_x, const float *d_y, int64_t rows, int cols)
 {
-	const int64_t groups = ((int64_t)cols + kCsCols - 1) / kCsCols;
+	anni_colsum job;
 
-	/* 63 row pitches must fit the 32-bit scalar offset of a buffer load */
-	if (!d_acc || !d_x || rows < 0 || cols <= 0 || cols > (1 << 24) || !device_ready())
-		return -1;
-	if (rows == 0)
-		return 0;
-	if (d_y)
-		hipLaunchKernelGGL((colsum_add_kernel<true>), dim3((unsigned)groups), dim3(kCsWaves * 64),
-		    0, compute_stream(), d_acc, d_x, d_y, rows, cols);
-	else
-		hipLaunchKernelGGL((colsum_add_kernel<false>), dim3((unsigned)groups),
-		    dim3(kCsWaves * 64), 0, compute_stream(), d_acc, d_x, d_y, rows, cols);
-	return hip_ok(hipGetLastError(), "colsum_add") ? 0 : -1;
+	job.d_acc = d_acc;
+	job.d_x = d_x;
+	job.d_y = d_y;
+	job.rows = rows;
+	job.cols = cols;
+	return anni_colsum_add_batch(&job, 1);
 }
 
 int anni_fp8_quantize(void *d_q, float *d_scale, const float *d_src, int64_t n)

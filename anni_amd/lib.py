@@ -44,6 +44,12 @@ class Adam(C.Structure):
                 ("d_pack_bf16", C.c_void_p), ("priv", C.c_void_p)]
 
 
+class Colsum(C.Structure):
+    """anni_colsum: one job of anni_colsum_add_batch."""
+    _fields_ = [("d_acc", C.c_void_p), ("d_x", C.c_void_p), ("d_y", C.c_void_p),
+                ("rows", C.c_int64), ("cols", C.c_int)]
+
+
 class Pack(C.Structure):
     """anni_pack: a second home for the bf16 of a matrix inside a packed matrix."""
     _fields_ = [("tensor", C.c_int), ("cols", C.c_int32), ("dst_offset", C.c_int64),
@@ -117,6 +123,7 @@ _PROTOS = {
     "anni_f32_to_bf16": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64]),
     "anni_fp8_quantize": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]),
     "anni_colsum_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]),
+    "anni_colsum_add_batch": (C.c_int, [C.POINTER(Colsum), C.c_int]),
 }
 
 _lib = None

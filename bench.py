@@ -219,6 +219,33 @@ def colsum_leg(L, rows, shapes=((6272, False), (1536, False), (1536, True))):
                     "ns_per_row": round(ms * 1e6 / rows, 2)})
         for b in (x, y, acc):
             b.free()
+    # the six sums of one 555M block (b1, b2, two LayerNorms) as one batch
+    from anni_amd import lib
+    shapes = [(6272, False), (1536, False), (1536, False), (1536, True), (1536, False), (1536, True)]
+    bufs, jobs = [], []
+    for k, (cols, prod) in enumerate(shapes):
+        n = rows * cols
+        x, y, acc = DeviceBuffer(n * 4), DeviceBuffer(n * 4 if prod else 4), DeviceBuffer(cols * 4)
+        assert L.anni_fill_normal_f32(x.ptr, n, 6, k, 0.0, 1e-2) == 0
+        if prod:
+            assert L.anni_fill_normal_f32(y.ptr, n, 7, k, 0.0, 1.0) == 0
+        assert L.gpu_memset(acc.ptr, 0, cols * 4) == 0
+        bufs += [x, y, acc]
+        jobs.append(lib.Colsum(acc.ptr, x.ptr, y.ptr if prod else None, rows, cols))
+    arr = (lib.Colsum * len(jobs))(*jobs)
+    for _ in range(3):
+        assert L.anni_colsum_add_batch(arr, len(jobs)) == 0
+    L.gpu_device_sync()
+    t0 = time.perf_counter()
+    for _ in range(20):
+        assert L.anni_colsum_add_batch(arr, len(jobs)) == 0
+    L.gpu_device_sync()
+    ms = (time.perf_counter() - t0) * 1e3 / 20
+    nbytes = sum(rows * c * 4 * (2 if p else 1) for c, p in shapes)
+    out.append({"batch": "b1 + b2 + 2 x (dbeta, dgamma) of one 555M block", "rows": rows,
+                "ms": round(ms, 4), "bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1)})
+    for b in bufs:
+        b.free()
     return out
 
 

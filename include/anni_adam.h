@@ -232,6 +232,20 @@ int	anni_fp8_quantize(void *d_q, float *d_scale, const float *d_src, int64_t n);
 ** rows == 0 leaves d_acc alone; cols up to 2^24.
 */
 int	anni_colsum_add(float *d_acc, const float *d_x, const float *d_y, int64_t rows, int cols);
+/*
+** Up to 16 such sums at once (the bias and LayerNorm gradients of a block, say): a sum narrower
+** than ~4000 columns occupies only cols / 64 of the 256 compute units, so sums launched one by
+** one leave most of the chip idle; here the plain sums share one launch and the product sums
+** another.  The jobs must not alias each other's d_acc.  Same results as one call per job.
+*/
+typedef struct anni_colsum {
+	float		*d_acc;
+	const float	*d_x;
+	const float	*d_y;	/* NULL: plain column sums */
+	int64_t		rows;
+	int		cols;
+} anni_colsum;
+int	anni_colsum_add_batch(const anni_colsum *jobs, int n_jobs);
 
 #ifdef __cplusplus
 }

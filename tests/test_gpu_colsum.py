@@ -124,6 +124,37 @@ def test_bias_gradient_lands_in_the_flat_and_the_step_uses_it(gpu, oracle):
     opt.free()
 
 
+def test_batch_equals_one_call_per_job(gpu, oracle):
+    """The bias and LayerNorm gradients of a block in one call: plain and product sums mixed,
+    widths that do not fill their last workgroup, a job without rows."""
+    from anni_amd import lib
+    from anni_amd.lm_adam import DeviceBuffer
+    rng = np.random.default_rng(99)
+    shapes = [(300, 6272, False), (300, 1536, False), (77, 1536, True), (300, 1, False),
+              (0, 64, False), (129, 1000, True), (64, 65, False), (1, 63, True)]
+    keep, jobs, want = [], [], []
+    for rows, cols, prod in shapes:
+        x, y, a0 = wide(rng, (rows, cols)), wide(rng, (rows, cols)), wide(rng, cols)
+        bufs = [DeviceBuffer(cols * 4), DeviceBuffer(max(x.nbytes, 4)), DeviceBuffer(max(y.nbytes, 4))]
+        bufs[0].upload(a0)
+        if rows:
+            bufs[1].upload(x)
+            bufs[2].upload(y)
+        keep.append(bufs)
+        jobs.append(lib.Colsum(bufs[0].ptr, bufs[1].ptr, bufs[2].ptr if prod else None, rows, cols))
+        want.append(oracle.colsum_add(a0.copy(), x, y if prod else None))
+    arr = (lib.Colsum * len(jobs))(*jobs)
+    assert gpu.anni_colsum_add_batch(arr, len(jobs)) == 0
+    for bufs, w in zip(keep, want):
+        assert same_bits(bufs[0].download(np.float32, w.size), w)
+    assert gpu.anni_colsum_add_batch(arr, 0) == -1
+    assert gpu.anni_colsum_add_batch(None, 1) == -1
+    assert gpu.anni_colsum_add_batch((lib.Colsum * 17)(*([jobs[0]] * 17)), 17) == -1
+    for bufs in keep:
+        for b in bufs:
+            b.free()
+
+
 def test_argument_checks(gpu):
     from anni_amd.lm_adam import DeviceBuffer
     d = DeviceBuffer(1024)
