@@ -97,7 +97,11 @@ __global__ __launch_bounds__(kThreads) void copy16_kernel(void *dst, const void 
 /* ---- column sums in the host loop's order ----------------------------------------- */
 
 constexpr int kCsCols = 64;		/* columns per workgroup: one per lane */
-constexpr int kCsWaves = 8;
+/*
+** Wavefronts per workgroup: eight turns cover the latency of the loads; 12 and 16 were measured
+** no faster (a narrow matrix is bound by the chain and the hand-over, ~5 ns a row, not by loads).
+*/
+template <bool PROD> struct CsWaves { static constexpr int n = 8; };
 /*
 ** Rows per chunk = what one wavefront holds in registers.  (With two matrices a chunk is 128
 ** loads, more than the 63 a wavefront can have outstanding, so that variant waits inside its
@@ -172,9 +176,10 @@ struct CsJobs {
 };
 
 template <bool PROD>
-__global__ __launch_bounds__(kCsWaves * 64) void colsum_add_kernel(CsJobs jobs)
+__global__ __launch_bounds__(CsWaves<PROD>::n * 64) void colsum_add_kernel(CsJobs jobs)
 {
 	constexpr int kCsRows = CsRows<PROD>::n;
+	constexpr int kCsWaves = CsWaves<PROD>::n;
 	__shared__ float carry[kCsCols];
 	const int lane = threadIdx.x & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -352,10 +357,10 @@ int anni_colsum_add_batch(const anni_colsum *jobs, int n_jobs)
 	}
 	if (plain.n)
 		hipLaunchKernelGGL((colsum_add_kernel<false>), dim3((unsigned)groups[0]),
-		    dim3(kCsWaves * 64), 0, compute_stream(), plain);
+		    dim3(CsWaves<false>::n * 64), 0, compute_stream(), plain);
 	if (prod.n)
 		hipLaunchKernelGGL((colsum_add_kernel<true>), dim3((unsigned)groups[1]),
-		    dim3(kCsWaves * 64), 0, compute_stream(), prod);
+		    dim3(CsWaves<true>::n * 64), 0, compute_stream(), prod);
 	return hip_ok(hipGetLastError(), "colsum_add") ? 0 : -1;
 }
 
