@@ -249,6 +249,36 @@ def colsum_leg(L, rows, shapes=((6272, False), (1536, False), (1536, True))):
     return out
 
 
+def ceilings(L, nbytes=8 << 30):
+    """What this box delivers to the simplest kernels of the library: write-only (fill), copy
+    (16-byte vectors, read + write) and read-only (the sum of squares), for comparison with the
+    update's mixed stream.  Every block sits in a 16 GiB region of its own."""
+    a, b = L.gpu_malloc(nbytes), L.gpu_malloc(nbytes)
+    assert a and b
+    assert L.gpu_memset(a, 1, nbytes) == 0 and L.gpu_memset(b, 0, nbytes) == 0
+    L.gpu_device_sync()
+
+    def timed(f, reps=10):
+        f()
+        L.gpu_device_sync()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            f()
+        L.gpu_device_sync()
+        return (time.perf_counter() - t0) / reps
+    ss = C.c_double(0)
+    n = min(nbytes // 4, (1 << 31) - 4096)
+    out = {"bytes": nbytes,
+           "write_only_GBps": round(nbytes / timed(lambda: L.gpu_memset(b, 3, nbytes)) / 1e9, 1),
+           "copy_read_plus_write_GBps":
+               round(2 * nbytes / timed(lambda: L.anni_copy_bytes(b, a, nbytes)) / 1e9, 1),
+           "read_only_GBps":
+               round(n * 4 / timed(lambda: L.gpu_grad_sumsq(a, n, C.byref(ss))) / 1e9, 1)}
+    L.gpu_free(a)
+    L.gpu_free(b)
+    return out
+
+
 def copy_calibration(L, nbytes):
     """Ten launches of the plain copy kernel: each reads nbytes and writes nbytes exactly."""
     from anni_amd.lm_adam import DeviceBuffer
@@ -277,6 +307,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="only run the plain copy kernel over BYTES ten times (counter calibration)")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="only measure write-only, copy and read-only throughput of the box")
     ap.add_argument("--colsum", type=int, default=0, metavar="ROWS",
                     help="only time the bias / LayerNorm gradient column sums over ROWS token rows")
     ap.add_argument("--reference-caller-only", action="store_true",
@@ -307,6 +339,9 @@ def main():
         env = bench_row.probe_env(L, os.path.dirname(os.path.abspath(__file__)))
     if a.copy_calibration:
         copy_calibration(L, a.copy_calibration)
+        return
+    if a.ceilings:
+        print(json.dumps({"ceilings": ceilings(L)}))
         return
     if a.colsum:
         print(json.dumps({"colsum_add": colsum_leg(L, a.colsum)}))
