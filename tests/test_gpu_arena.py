@@ -337,3 +337,44 @@ def test_device_normal_generator_and_bf16_convert(gpu, oracle):
     h = DeviceBuffer(n * 2)
     assert gpu.anni_f32_to_bf16(h.ptr, a.ptr, n) == 0
     assert (h.download(np.uint16, n) == oracle.bf16_rne(x)).all()
+
+
+def test_two_optimizers_side_by_side(gpu, oracle):
+    """Two arenas with different storage modes stepping in turn share the stream and the
+    library's state and do not disturb each other."""
+    rng = np.random.default_rng(77)
+    a = make(gpu, RAGGED, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True)
+    b = make(gpu, [(9000, 3), (17, 0)], grad_type=BF16, moment_type=BF16, beta2=0.99,
+             weight_decay=0.01, grad_clip=0.5)
+    st = {}
+    for opt, name in ((a, "a"), (b, "b")):
+        n = opt.n
+        p = (rng.standard_normal(n) * 0.02).astype(np.float32)
+        opt.upload("param", p)
+        opt.seed_twins()
+        bf = name == "b"
+        st[name] = dict(P=p.copy(), M=np.zeros(n, np.uint16 if bf else np.float32),
+                        V=np.zeros(n, np.uint16 if bf else np.float32),
+                        O=oracle.Oracle(n, beta2=0.99 if bf else 0.95,
+                                        weight_decay=0.01 if bf else 0.1,
+                                        grad_clip=0.5 if bf else 1.0, skip_nonfinite=not bf,
+                                        grad_type=oracle.BF16 if bf else oracle.F32,
+                                        moment_type=oracle.BF16 if bf else oracle.F32,
+                                        tensors=oracle_tensors(opt), threads=2))
+    for s in range(4):
+        grads = {}
+        for opt, name in ((a, "a"), (b, "b")):
+            g = (rng.standard_normal(opt.n) * (3e-2 if s % 2 else 1e-4)).astype(np.float32)
+            grads[name] = oracle.bf16_rne(g) if name == "b" else g
+            opt.upload("grad", grads[name])
+        assert a.step_scaled(1e-3) == 0 and b.step_scaled(2e-3) == 0       # both queued, then read
+        for opt, name, lr in ((a, "a", 1e-3), (b, "b", 2e-3)):
+            stats = opt.sync_stats()
+            S = st[name]
+            S["O"].step(S["P"], grads[name].copy(), S["M"], S["V"], lr,
+                        sumsq_override=stats.last_sumsq)
+            assert stats.last_clipped == S["O"].o.last_clipped == s % 2
+            assert same_bits(opt.download("param"), S["P"]), (name, s)
+            assert (opt.download("m") == S["M"]).all() and (opt.download("v") == S["V"]).all()
+    a.free()
+    b.free()
