@@ -305,6 +305,7 @@ static anni_adam *create_body(const anni_tensor *tensors, int n_tensors,
 
 	if (!tensors || n_tensors <= 0 || !cfg || !device_ready())
 		return nullptr;
+	(void)release_idle_slab();	/* the arena's own reservation is sized by what is free */
 	if (cfg->grad_type < ANNI_F32 || cfg->grad_type > ANNI_FP8_E4M3
 	    || (cfg->moment_type != ANNI_F32 && cfg->moment_type != ANNI_BF16)
 	    || cfg->grad_slots < 0 || cfg->grad_slots > 4096

@@ -17,6 +17,11 @@ hipStream_t	compute_stream(void);
 void		set_compute_stream(hipStream_t st);
 /* Remembers the first HIP error for gpu_debug_last_error; returns err == hipSuccess. */
 bool		hip_ok(hipError_t err, const char *what);
+/*
+** gpu_malloc keeps its region slab reserved after the last block in it was freed; this gives it
+** back to the driver (true when there was one).  Called before other large reservations.
+*/
+bool		release_idle_slab(void);
 
 } /* namespace anni */
 #endif

@@ -379,6 +379,8 @@ const char *gpu_backend_name(void)
 	return "hip-gfx950";
 }
 
+static size_t slab_idle_bytes_locked(void);
+
 int gpu_mem_info(size_t *free_bytes, size_t *total_bytes)
 {
 	size_t f = 0;
@@ -386,6 +388,11 @@ int gpu_mem_info(size_t *free_bytes, size_t *total_bytes)
 
 	if (!device_ready() || !hip_ok(hipMemGetInfo(&f, &t), "hipMemGetInfo"))
 		return -1;
+	{
+		std::lock_guard<std::mutex> lk(g_mu);
+
+		f += slab_idle_bytes_locked();	/* reserved, but given back on demand */
+	}
 	if (free_bytes)
 		*free_bytes = f;
 	if (total_bytes)
@@ -473,6 +480,10 @@ void gpu_op_prof_dump(void)
 ** puts the caller's p, g, twin, m, v where the arena of anni_adam_create puts them (three
 ** flats per 64 GiB group).  Anything that does not fit (no free region, larger than a
 ** region, slab not available) is a plain hipMalloc.  ANNI_MALLOC_SPREAD=0 switches it off.
+** A slab whose last region was returned stays reserved (reserving and releasing 96 GiB costs
+** the driver about a second, and a caller that frees and re-allocates its flats would pay it
+** every time) until memory is wanted elsewhere: an allocation that fails, or an arena being
+** created, releases it first; gpu_mem_info counts it as free.
 */
 static const size_t kSpreadMin = (size_t)256 << 20;
 static const size_t kRegion = (size_t)16 << 30;
@@ -535,13 +546,25 @@ static bool spread_give(void *p)
 	if (off % kRegion != 0 || !g_region_used[off / kRegion])
 		return false;
 	g_region_used[off / kRegion] = false;
-	if (--g_regions_live == 0) {
-		/* Last region returned: give the slab back and start over on the next large request. */
-		(void)hipStreamSynchronize(g_stream);
-		(void)hipFree(g_slab);
-		g_slab = nullptr;
-		g_slab_tried = false;
-	}
+	g_regions_live--;
+	return true;
+}
+
+/* Called with g_mu held.  Size of a slab that is reserved but holds no block. */
+static size_t slab_idle_bytes_locked(void)
+{
+	return g_slab && g_regions_live == 0 ? (size_t)kSpreadRegions * kRegion : 0;
+}
+
+/* Called with g_mu held.  Gives an unused slab back to the driver; true when it did. */
+static bool slab_release_idle_locked(void)
+{
+	if (!g_slab || g_regions_live != 0)
+		return false;
+	(void)hipStreamSynchronize(g_stream);
+	(void)hipFree(g_slab);
+	g_slab = nullptr;
+	g_slab_tried = false;
 	return true;
 }
 
@@ -558,9 +581,21 @@ void *gpu_malloc(size_t nbytes)
 	}
 	if (p)
 		return p;
-	if (!hip_ok(hipMalloc(&p, nbytes), "hipMalloc")) {
+	if (hipMalloc(&p, nbytes) != hipSuccess) {
+		bool released;
+
 		(void)hipGetLastError();
-		return nullptr;
+		{
+			std::lock_guard<std::mutex> lk(g_mu);
+
+			released = slab_release_idle_locked();
+		}
+		if (!released || !hip_ok(hipMalloc(&p, nbytes), "hipMalloc")) {
+			if (!released)
+				(void)hip_ok(hipErrorOutOfMemory, "hipMalloc");
+			(void)hipGetLastError();
+			return nullptr;
+		}
 	}
 	return p;
 }
@@ -796,3 +831,14 @@ int gpu_adam_step_dev_bf16(ann_real *d_param, void *d_param_bf16, ann_real *d_gr
 }
 
 } /* extern "C" */
+
+namespace anni {
+
+bool release_idle_slab(void)
+{
+	std::lock_guard<std::mutex> lk(g_mu);
+
+	return slab_release_idle_locked();
+}
+
+} /* namespace anni */

@@ -372,11 +372,23 @@ def test_large_allocations_are_spread_over_regions(gpu):
     assert gpu.gpu_memset(ptrs[3], 0x5a, 4 * n) == 0
     tail = np.zeros(16, np.uint8)
     assert gpu.gpu_memcpy_d2h(tail.ctypes.data, ptrs[3] + 4 * n - 16, 16) == 0 and (tail == 0x5a).all()
+    fr_live, fr_idle, tt = C.c_size_t(0), C.c_size_t(0), C.c_size_t(0)
+    assert gpu.gpu_mem_info(C.byref(fr_live), C.byref(tt)) == 0
     for p in [ptrs[0], again, ptrs[2], ptrs[3], ptrs[4], small]:
         gpu.gpu_free(p)
-    fresh = gpu.gpu_malloc(4 * n)                        # everything returned: a new slab next time
-    assert fresh
+    # everything returned: the slab stays reserved for the next large request (no driver round
+    # trip), is reported as free memory, and goes back to the driver when an arena is created
+    assert gpu.gpu_mem_info(C.byref(fr_idle), C.byref(tt)) == 0
+    assert fr_idle.value >= fr_live.value + (6 << 34)
+    fresh = gpu.gpu_malloc(4 * n)
+    assert fresh == base
     gpu.gpu_free(fresh)
+    from anni_amd.lm_adam import LmAdam
+    opt = LmAdam([(4096, 3)])
+    opt.free()
+    again2 = gpu.gpu_malloc(4 * n)                       # a new slab after the release
+    assert again2
+    gpu.gpu_free(again2)
 
 
 def test_small_copies_are_batched_in_order(gpu):
@@ -421,3 +433,45 @@ def test_small_copies_are_batched_in_order(gpu):
     for off, ln, o in outs:
         assert (o == ref[off:off + ln]).all(), (off, ln)
     assert not d.download(np.uint8, 4096).any()
+
+
+def test_malloc_and_free_from_many_threads(gpu):
+    """gpu_malloc / gpu_free are called from OpenMP threads in the reference (gpu_cuda.cu:2644-2645):
+    eight threads allocate, fill, check and free blocks of mixed sizes, the large ones out of the
+    region slab; afterwards the device holds what it held before."""
+    import threading
+    fr0, tt = C.c_size_t(0), C.c_size_t(0)
+    hold = gpu.gpu_malloc(300 << 20)                 # keeps the region slab alive while the threads churn
+    assert hold
+    gpu.gpu_device_sync()
+    assert gpu.gpu_mem_info(C.byref(fr0), C.byref(tt)) == 0
+    errors = []
+
+    def worker(k):
+        try:
+            rng = np.random.default_rng(k)
+            for i in range(25):
+                nbytes = int(rng.choice([64, 4096, 1 << 20, 300 << 20])) + 16 * int(rng.integers(0, 8))
+                p = gpu.gpu_malloc(nbytes)
+                if not p:
+                    raise MemoryError(nbytes)
+                val = (k * 25 + i) % 251 + 1
+                if gpu.gpu_memset(p, val, min(nbytes, 1 << 16)) != 0:
+                    raise RuntimeError("memset")
+                out = np.zeros(64, np.uint8)
+                if gpu.gpu_memcpy_d2h(out.ctypes.data, p, 64) != 0 or not (out == val).all():
+                    raise RuntimeError("thread %d block %d read back %r" % (k, i, out[:4]))
+                gpu.gpu_free(p)
+        except Exception as e:                       # noqa: BLE001 - reported below
+            errors.append(repr(e))
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    gpu.gpu_device_sync()
+    fr1 = C.c_size_t(0)
+    assert gpu.gpu_mem_info(C.byref(fr1), C.byref(tt)) == 0
+    assert abs(fr1.value - fr0.value) <= 64 << 20    # the runtime's own pools may have grown a little
+    gpu.gpu_free(hold)
