@@ -748,10 +748,8 @@ __global__ __launch_bounds__(kThreads) void fp8_twin_kernel(Fp8TwinArgs a)
 				P[u] = load_quad<kF32, NT>(a.p, base + (int64_t)(u * kThreads + tid) * kQuad, 1.0f);
 #pragma unroll
 			for (int u = 0; u < kQuadsPerTile; u++) {
-				const uint32_t w = fp8_e4m3_encode(P[u].x * inv)
-				    | (fp8_e4m3_encode(P[u].y * inv) << 8)
-				    | (fp8_e4m3_encode(P[u].z * inv) << 16)
-				    | (fp8_e4m3_encode(P[u].w * inv) << 24);
+				const uint32_t w = fp8_e4m3_encode4(P[u].x * inv, P[u].y * inv, P[u].z * inv,
+				    P[u].w * inv);
 
 				st<NT>((uint32_t *)(a.q + base + (int64_t)(u * kThreads + tid) * kQuad), w);
 			}

@@ -143,6 +143,36 @@ __device__ __forceinline__ uint32_t fp8_e4m3_encode(float x)
 }
 
 /*
+** Four floats -> four OCP E4M3 bytes (x in the low byte) with the gfx950 conversion instruction:
+** round to nearest even on the format's grid, subnormals included.  The instruction alone would
+** turn an overflow into NaN, so the values are first clamped to +-448 (an infinity saturates);
+** a NaN input is patched to S.1111.111 afterwards, whatever the clamp made of it.  Same bytes as
+** fp8_e4m3_encode on every input (checked on every rounding boundary of the format).
+*/
+__device__ __forceinline__ uint32_t fp8_e4m3_encode4(float x, float y, float z, float w)
+{
+	const float lim = 448.0f;
+	int r = __builtin_amdgcn_cvt_pk_fp8_f32(__builtin_amdgcn_fmed3f(x, -lim, lim),
+	    __builtin_amdgcn_fmed3f(y, -lim, lim), 0, false);
+	uint32_t out;
+
+	r = __builtin_amdgcn_cvt_pk_fp8_f32(__builtin_amdgcn_fmed3f(z, -lim, lim),
+	    __builtin_amdgcn_fmed3f(w, -lim, lim), r, true);
+	out = (uint32_t)r;
+	if (x != x || y != y || z != z || w != w) {
+		if (x != x)
+			out = (out & 0xffffff00u) | ((__float_as_uint(x) >> 24) & 0x80u) | 0x7fu;
+		if (y != y)
+			out = (out & 0xffff00ffu) | ((((__float_as_uint(y) >> 24) & 0x80u) | 0x7fu) << 8);
+		if (z != z)
+			out = (out & 0xff00ffffu) | ((((__float_as_uint(z) >> 24) & 0x80u) | 0x7fu) << 16);
+		if (w != w)
+			out = (out & 0x00ffffffu) | ((((__float_as_uint(w) >> 24) & 0x80u) | 0x7fu) << 24);
+	}
+	return out;
+}
+
+/*
 ** Per-tensor FP8 scale from the tensor's max |x| (num/gpu_cuda.cu:927-938): amax / 448, at
 ** least 1e-12; a zero, negative or non-finite amax counts as 1e-8.
 */

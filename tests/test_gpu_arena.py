@@ -378,3 +378,42 @@ def test_two_optimizers_side_by_side(gpu, oracle):
             assert (opt.download("m") == S["M"]).all() and (opt.download("v") == S["V"]).all()
     a.free()
     b.free()
+
+
+def test_fp8_quantizer_on_every_rounding_boundary(gpu, oracle):
+    """The device quantiser against the oracle's (pinned to torch's float8_e4m3fn cast) on a tensor
+    whose amax is exactly 448, so the scale is 1 and the bytes are the plain encoding of the
+    inputs: for every binade of the format, both signs and every half step of its 3-bit mantissa,
+    the tie itself and its two float neighbours; the subnormal grid; 448 and just below; signed
+    zeros; float denormals; and two million random values."""
+    from anni_amd.lm_adam import DeviceBuffer
+    vals = [448.0, 0.0, -0.0, 1e-45, -1e-45, 1e-39, 2.0 ** -10, 2.0 ** -9, 3 * 2.0 ** -10,
+            447.99997, 432.0, 464.0 - 32.0, 2.0 ** -6, 2.0 ** -7, 0.0146484375]
+    for e in range(-12, 9):
+        for k in range(0, 32):                         # 1.k/16 * 2^e: grid points and ties
+            c = np.float32((1.0 + k / 16.0) * 2.0 ** e)
+            if c > 448:
+                continue
+            for v in (c, np.nextafter(c, np.float32(0)), np.nextafter(c, np.float32(1e9))):
+                if v <= 448:
+                    vals += [float(v), -float(v)]
+    rng = np.random.default_rng(123)
+    rnd = (rng.standard_normal(2000000) * 10.0 ** rng.integers(-6, 3, 2000000)).astype(np.float32)
+    x = np.concatenate([np.array(vals, np.float32), np.clip(rnd, -448, 448)])
+    assert np.abs(x).max() == 448.0
+    src, q, sc = DeviceBuffer(x.nbytes), DeviceBuffer(x.size), DeviceBuffer(4)
+    src.upload(x)
+    assert gpu.anni_fp8_quantize(q.ptr, sc.ptr, src.ptr, x.size) == 0
+    assert gpu.gpu_stream_sync() == 0
+    want, scale = oracle.fp8_quantize(x)
+    assert scale == 1.0 and sc.download(np.float32, 1)[0] == 1.0
+    got = q.download(np.uint8, x.size)
+    bad = np.flatnonzero(got != want)
+    assert bad.size == 0, [(float(x[i]), int(got[i]), int(want[i])) for i in bad[:8]]
+    # non-finite inputs: the amax is then taken as 1e-8 (scale 1e-8/448), NaN stays NaN, infinities saturate
+    y = np.array([np.nan, -np.nan, np.inf, -np.inf, 1e-9, -3e-9, 0.0], np.float32)
+    src.upload(y)
+    assert gpu.anni_fp8_quantize(q.ptr, sc.ptr, src.ptr, y.size) == 0
+    assert gpu.gpu_stream_sync() == 0
+    want, scale = oracle.fp8_quantize(y)
+    assert (q.download(np.uint8, y.size) == want).all() and sc.download(np.float32, 1)[0] == scale

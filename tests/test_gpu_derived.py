@@ -257,3 +257,43 @@ def test_185m_reference_layout_full_size(gpu, oracle):
         assert (opt.download("pack") == pk).all(), s
         print("185m derived step %d ok" % (s + 1), flush=True)
     opt.free()
+
+
+def test_hardware_encode_on_every_rounding_boundary(gpu, oracle):
+    """The E4M3 twins of whole tiles are made with the gfx950 conversion instruction, the ragged
+    ends with the bit-level encoder: both against the oracle's encoder (pinned to torch's
+    float8_e4m3fn cast) on tensors whose max |p| is exactly 448, so scale = 1 and the bytes are the
+    plain encoding: every binade, both signs, every half step of the 3-bit mantissa with its two
+    float neighbours, the subnormal grid, signed zeros, float denormals, NaNs of both signs,
+    and random values."""
+    vals = [448.0, 0.0, -0.0, 1e-45, -1e-45, 1e-39, 2.0 ** -10, 2.0 ** -9, 3 * 2.0 ** -10,
+            447.99997, 432.0, 2.0 ** -6, 2.0 ** -7, 0.0146484375, np.nan, -np.nan]
+    for e in range(-12, 9):
+        for k in range(0, 32):
+            c = np.float32((1.0 + k / 16.0) * 2.0 ** e)
+            if c > 448:
+                continue
+            for v in (c, np.nextafter(c, np.float32(0)), np.nextafter(c, np.float32(1e9))):
+                if v <= 448:
+                    vals += [float(v), -float(v)]
+    rng = np.random.default_rng(321)
+    n_big = 4096 * 40
+    rnd = (rng.standard_normal(n_big) * 10.0 ** rng.integers(-6, 3, n_big)).astype(np.float32)
+    big = np.clip(rnd, -448, 448)
+    special = np.array(vals, np.float32)
+    big[:special.size] = special                       # whole tiles: the hardware path
+    big = big[rng.permutation(n_big)]
+    tail = np.concatenate([special, np.float32([448.0])])[:4095]     # a ragged tensor: the bit-level path
+    opt = make([(n_big, FP8TWIN), (tail.size, FP8TWIN)], twins=False)
+    opt.upload("param", np.concatenate([big, tail]))
+    opt.enable_derived()
+    opt.seed_twins()
+    got, sc = opt.download("fp8twin"), opt.download("wscale")
+    assert sc[0] == 1.0 and sc[1] == 1.0
+    for off, x in ((0, big), (n_big, tail)):
+        want, scale = oracle.fp8_quantize(x)
+        assert scale == 1.0
+        g = got[off:off + x.size]
+        bad = np.flatnonzero(g != want)
+        assert bad.size == 0, [(float(x[i]), int(g[i]), int(want[i])) for i in bad[:8]]
+    opt.free()
