@@ -876,27 +876,37 @@ int anni_adam_time_steps(anni_adam *opt, int count, void *const *grads, int n_gr
 /* Slots per staging round: the reference's ADAM_CHUNK (lm_serialize.c:261), 16 MiB of pairs. */
 static const int64_t kCkptChunk = (int64_t)1 << 21;
 
-/* Two page-locked + two device staging buffers of one chunk each, for the lifetime of one call. */
+/*
+** Two page-locked + two device staging buffers of one chunk each and an event per buffer, for
+** the lifetime of one call.
+*/
 struct CkptStage {
-	float	*host[2];
-	float	*dev[2];
+	float		*host[2];
+	float		*dev[2];
+	hipEvent_t	ev[2];
+	bool		have_ev[2];
 
-	CkptStage() : host{nullptr, nullptr}, dev{nullptr, nullptr} {}
+	CkptStage() : host{nullptr, nullptr}, dev{nullptr, nullptr}, ev{}, have_ev{false, false} {}
 	bool init(void)
 	{
 		const size_t bytes = (size_t)kCkptChunk * 2 * sizeof(float);
 
-		for (int i = 0; i < 2; i++)
+		for (int i = 0; i < 2; i++) {
 			if (hipHostMalloc((void **)&host[i], bytes, hipHostMallocDefault) != hipSuccess
-			    || hipMalloc((void **)&dev[i], bytes) != hipSuccess) {
+			    || hipMalloc((void **)&dev[i], bytes) != hipSuccess
+			    || hipEventCreateWithFlags(&ev[i], hipEventDisableTiming) != hipSuccess) {
 				(void)hipGetLastError();
 				return false;
 			}
+			have_ev[i] = true;
+		}
 		return true;
 	}
 	~CkptStage()
 	{
 		for (int i = 0; i < 2; i++) {
+			if (have_ev[i])
+				(void)hipEventDestroy(ev[i]);
 			if (host[i])
 				(void)hipHostFree(host[i]);
 			if (dev[i])
@@ -905,50 +915,74 @@ struct CkptStage {
 	}
 };
 
-int anni_adam_export_mv(anni_adam *opt, int64_t first, int64_t count, float *pairs)
+/* Where exported pairs go / imported pairs come from: a host array or a file descriptor. */
+struct PairIo {
+	float	*mem;		/* NULL: use fd */
+	int	fd;
+};
+
+static int write_all(int fd, const void *buf, size_t n);
+static int read_all(int fd, void *buf, size_t n);
+
+/*
+** Slots [first, first + count) as (m, v) pairs, chunk by chunk: while the host consumes chunk k
+** out of one page-locked buffer (a copy into the caller's array, or write(2) straight from the
+** buffer) the device interleaves chunk k + 1 and sends it into the other.
+*/
+static int export_pairs(anni_adam *opt, int64_t first, int64_t count, const PairIo &io)
 {
 	hipStream_t st;
 	CkptStage sg;
-	int rc = 0;
+	const int64_t n_chunks = (count + kCkptChunk - 1) / kCkptChunk;
 
-	if (!opt || !opt->priv || !pairs || first < 0 || count < 0 || first + count > opt->n
-	    || !device_ready())
-		return -1;
 	if (count == 0)
 		return 0;
 	if (!sg.init())
 		return -1;
 	st = compute_stream();
-	for (int64_t at = 0, k = 0; rc == 0; at += kCkptChunk, k++) {
-		const int64_t c = count - at < kCkptChunk ? count - at : kCkptChunk;
-		const int b = (int)(k & 1);
+	for (int64_t k = -1; k < n_chunks; k++) {
+		if (k + 1 < n_chunks) {		/* issue chunk k + 1 */
+			const int64_t at = (k + 1) * kCkptChunk;
+			const int64_t c = count - at < kCkptChunk ? count - at : kCkptChunk;
+			const int b = (int)((k + 1) & 1);
 
-		if (c > 0) {
 			if (launch_mv_interleave(st, sg.dev[b], opt->d_m, opt->d_v, opt->cfg.moment_type,
 			    first + at, c) != 0
 			    || !hip_ok(hipMemcpyAsync(sg.host[b], sg.dev[b], (size_t)c * 2 * sizeof(float),
-			    hipMemcpyDeviceToHost, st), "export_mv d2h"))
-				rc = -1;
+			    hipMemcpyDeviceToHost, st), "export d2h")
+			    || !hip_ok(hipEventRecord(sg.ev[b], st), "export event")) {
+				(void)hipStreamSynchronize(st);
+				return -1;
+			}
 		}
-		if (rc == 0 && !hip_ok(hipStreamSynchronize(st), "export_mv sync"))
-			rc = -1;
-		if (rc == 0 && c > 0)
-			memcpy(pairs + 2 * at, sg.host[b], (size_t)c * 2 * sizeof(float));
-		if (at + kCkptChunk >= count)
-			break;
+		if (k >= 0) {			/* consume chunk k */
+			const int64_t at = k * kCkptChunk;
+			const int64_t c = count - at < kCkptChunk ? count - at : kCkptChunk;
+			const int b = (int)(k & 1);
+			const size_t bytes = (size_t)c * 2 * sizeof(float);
+
+			if (!hip_ok(hipEventSynchronize(sg.ev[b]), "export wait")) {
+				(void)hipStreamSynchronize(st);
+				return -1;
+			}
+			if (io.mem)
+				memcpy(io.mem + 2 * at, sg.host[b], bytes);
+			else if (write_all(io.fd, sg.host[b], bytes) != 0) {
+				(void)hipStreamSynchronize(st);
+				return -1;
+			}
+		}
 	}
-	return rc;
+	return 0;
 }
 
-int anni_adam_import_mv(anni_adam *opt, int64_t first, int64_t count, const float *pairs)
+/* The other way: the host fills one page-locked buffer while the device scatters the other. */
+static int import_pairs(anni_adam *opt, int64_t first, int64_t count, const PairIo &io)
 {
 	hipStream_t st;
 	CkptStage sg;
 	int rc = 0;
 
-	if (!opt || !opt->priv || !pairs || first < 0 || count < 0 || first + count > opt->n
-	    || !device_ready())
-		return -1;
 	if (count == 0)
 		return 0;
 	if (!sg.init())
@@ -957,22 +991,51 @@ int anni_adam_import_mv(anni_adam *opt, int64_t first, int64_t count, const floa
 	for (int64_t at = 0, k = 0; at < count && rc == 0; at += kCkptChunk, k++) {
 		const int64_t c = count - at < kCkptChunk ? count - at : kCkptChunk;
 		const int b = (int)(k & 1);
+		const size_t bytes = (size_t)c * 2 * sizeof(float);
 
-		/* buffer b was last used two chunks ago: wait before overwriting it */
-		if (k >= 2 && !hip_ok(hipStreamSynchronize(st), "import_mv sync"))
+		/* buffer b was last used two chunks ago: its upload must be over before it is refilled */
+		if (k >= 2 && !hip_ok(hipEventSynchronize(sg.ev[b]), "import wait"))
 			rc = -1;
 		if (rc == 0) {
-			memcpy(sg.host[b], pairs + 2 * at, (size_t)c * 2 * sizeof(float));
-			if (!hip_ok(hipMemcpyAsync(sg.dev[b], sg.host[b], (size_t)c * 2 * sizeof(float),
-			    hipMemcpyHostToDevice, st), "import_mv h2d")
-			    || launch_mv_deinterleave(st, opt->d_m, opt->d_v, opt->cfg.moment_type,
-			    sg.dev[b], first + at, c) != 0)
+			if (io.mem)
+				memcpy(sg.host[b], io.mem + 2 * at, bytes);
+			else if (read_all(io.fd, sg.host[b], bytes) != 0)
 				rc = -1;
 		}
+		if (rc == 0 && (!hip_ok(hipMemcpyAsync(sg.dev[b], sg.host[b], bytes, hipMemcpyHostToDevice,
+		    st), "import h2d")
+		    || launch_mv_deinterleave(st, opt->d_m, opt->d_v, opt->cfg.moment_type, sg.dev[b],
+		    first + at, c) != 0
+		    || !hip_ok(hipEventRecord(sg.ev[b], st), "import event")))
+			rc = -1;
 	}
-	if (!hip_ok(hipStreamSynchronize(st), "import_mv sync"))
+	if (!hip_ok(hipStreamSynchronize(st), "import sync"))
 		rc = -1;
 	return rc;
+}
+
+int anni_adam_export_mv(anni_adam *opt, int64_t first, int64_t count, float *pairs)
+{
+	PairIo io;
+
+	if (!opt || !opt->priv || !pairs || first < 0 || count < 0 || first + count > opt->n
+	    || !device_ready())
+		return -1;
+	io.mem = pairs;
+	io.fd = -1;
+	return export_pairs(opt, first, count, io);
+}
+
+int anni_adam_import_mv(anni_adam *opt, int64_t first, int64_t count, const float *pairs)
+{
+	PairIo io;
+
+	if (!opt || !opt->priv || !pairs || first < 0 || count < 0 || first + count > opt->n
+	    || !device_ready())
+		return -1;
+	io.mem = const_cast<float *>(pairs);
+	io.fd = -1;
+	return import_pairs(opt, first, count, io);
 }
 
 static int write_all(int fd, const void *buf, size_t n)
@@ -1008,10 +1071,9 @@ static int read_all(int fd, void *buf, size_t n)
 int anni_adam_write_state(anni_adam *opt, int fd, int epoch, int step)
 {
 	int32_t head[5];
-	float *buf;
-	int rc = 0;
+	PairIo io;
 
-	if (!opt || !opt->priv || fd < 0 || opt->n > INT32_MAX)
+	if (!opt || !opt->priv || fd < 0 || opt->n > INT32_MAX || !device_ready())
 		return -1;
 	head[0] = 1;			/* lm_serialize.c:319-321: has_adam, epoch, step, t, n */
 	head[1] = epoch;
@@ -1020,43 +1082,24 @@ int anni_adam_write_state(anni_adam *opt, int fd, int epoch, int step)
 	head[4] = (int32_t)opt->n;
 	if (write_all(fd, head, sizeof(head)) != 0)
 		return -1;
-	buf = (float *)malloc((size_t)kCkptChunk * 2 * sizeof(float));
-	if (!buf)
-		return -1;
-	for (int64_t at = 0; at < opt->n && rc == 0; at += kCkptChunk) {
-		const int64_t c = opt->n - at < kCkptChunk ? opt->n - at : kCkptChunk;
-
-		if (anni_adam_export_mv(opt, at, c, buf) != 0
-		    || write_all(fd, buf, (size_t)c * 2 * sizeof(float)) != 0)
-			rc = -1;
-	}
-	free(buf);
-	return rc;
+	io.mem = nullptr;
+	io.fd = fd;
+	return export_pairs(opt, 0, opt->n, io);	/* write(2) straight from the page-locked buffers */
 }
 
 int anni_adam_read_state(anni_adam *opt, int fd, int *epoch, int *step)
 {
 	int32_t head[5];
-	float *buf;
-	int rc = 0;
+	PairIo io;
 
-	if (!opt || !opt->priv || fd < 0)
+	if (!opt || !opt->priv || fd < 0 || !device_ready())
 		return -1;
 	if (read_all(fd, head, sizeof(head)) != 0 || head[0] != 1 || head[4] != opt->n)
 		return -1;		/* lm_serialize.c:546-562: has_adam == 1 and the same slot count */
-	buf = (float *)malloc((size_t)kCkptChunk * 2 * sizeof(float));
-	if (!buf)
-		return -1;
-	for (int64_t at = 0; at < opt->n && rc == 0; at += kCkptChunk) {
-		const int64_t c = opt->n - at < kCkptChunk ? opt->n - at : kCkptChunk;
-
-		if (read_all(fd, buf, (size_t)c * 2 * sizeof(float)) != 0
-		    || anni_adam_import_mv(opt, at, c, buf) != 0)
-			rc = -1;
-	}
-	free(buf);
-	if (rc != 0)
-		return -1;
+	io.mem = nullptr;
+	io.fd = fd;
+	if (import_pairs(opt, 0, opt->n, io) != 0)
+		return -1;		/* a short file: the moments read so far are in place, t is not */
 	opt->t = head[3];		/* so the learning-rate schedule continues (lm_serialize.c:564) */
 	if (epoch)
 		*epoch = head[1];

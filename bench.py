@@ -249,6 +249,43 @@ def colsum_leg(L, rows, shapes=((6272, False), (1536, False), (1536, True))):
     return out
 
 
+def ckpt_leg(L, size="555m"):
+    """The optimizer block of a checkpoint (has_adam, epoch, step, t, n + n interleaved (m, v)
+    pairs) written from and read into the arena: to /dev/null (device side + host link alone)
+    and through a file on tmpfs."""
+    import tempfile
+    from anni_amd import layout
+    from anni_amd.lm_adam import LmAdam
+    opt = LmAdam(layout.tensors(size), twins=False, grad_slots=1)
+    n = opt.n
+    assert L.anni_fill_normal_f32(opt.o.d_m, n, 8, 1, 0.0, 1e-3) == 0
+    assert L.anni_fill_normal_f32(opt.o.d_v, n, 8, 2, 1e-6, 1e-7) == 0
+    L.gpu_device_sync()
+    nbytes = 20 + 8 * n
+    out = {"workload": size, "slots": n, "block_bytes": nbytes}
+    fd = os.open("/dev/null", os.O_WRONLY)
+    opt.write_state(fd, 1, 2)                                       # warm the staging buffers
+    t0 = time.perf_counter()
+    opt.write_state(fd, 1, 2)
+    dt = time.perf_counter() - t0
+    os.close(fd)
+    out["write_to_devnull"] = {"ms": round(dt * 1e3, 1), "GBps": round(nbytes / dt / 1e9, 2)}
+    d = "/dev/shm" if os.path.isdir("/dev/shm") else None
+    with tempfile.NamedTemporaryFile(dir=d) as f:
+        t0 = time.perf_counter()
+        opt.write_state(f.fileno(), 1, 2)
+        dt = time.perf_counter() - t0
+        out["write_to_tmpfs"] = {"ms": round(dt * 1e3, 1), "GBps": round(nbytes / dt / 1e9, 2)}
+        os.lseek(f.fileno(), 0, os.SEEK_SET)
+        t0 = time.perf_counter()
+        opt.read_state(f.fileno())
+        L.gpu_device_sync()
+        dt = time.perf_counter() - t0
+        out["read_from_tmpfs"] = {"ms": round(dt * 1e3, 1), "GBps": round(nbytes / dt / 1e9, 2)}
+    opt.free()
+    return out
+
+
 def ceilings(L, nbytes=8 << 30):
     """What this box delivers to the simplest kernels of the library: write-only (fill), copy
     (16-byte vectors, read + write) and read-only (the sum of squares), for comparison with the
@@ -307,6 +344,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="only run the plain copy kernel over BYTES ten times (counter calibration)")
+    ap.add_argument("--ckpt", action="store_true",
+                    help="only time the optimizer block of a checkpoint written from / read into the arena")
     ap.add_argument("--ceilings", action="store_true",
                     help="only measure write-only, copy and read-only throughput of the box")
     ap.add_argument("--colsum", type=int, default=0, metavar="ROWS",
@@ -339,6 +378,9 @@ def main():
         env = bench_row.probe_env(L, os.path.dirname(os.path.abspath(__file__)))
     if a.copy_calibration:
         copy_calibration(L, a.copy_calibration)
+        return
+    if a.ckpt:
+        print(json.dumps({"checkpoint_block": ckpt_leg(L)}))
         return
     if a.ceilings:
         print(json.dumps({"ceilings": ceilings(L)}))
