@@ -45,10 +45,9 @@ struct anni_adam_priv {
 	std::vector<Seg>	segs;		/* host copy of the device table */
 	void			*derived;
 	int			derived_owned;	/* 1: derived is an allocation of its own */
-	uint32_t		*d_wamax[2];	/* this step's and the next step's max |p| words */
+	uint32_t		*d_wamax;	/* max |p| of each flagged tensor, cleared by a fill kernel before every step */
 	PackDesc		*d_packs;
 	float			*d_tile_amax;	/* per-wavefront max |p| of every whole tile */
-	int			der_cur;	/* which of d_wamax the next producer raises */
 	int			fp8_twins;	/* 1: some tensor keeps an E4M3 twin */
 	float			der_ms;		/* E4M3 pass time summed by anni_adam_time_steps */
 };
@@ -521,16 +520,17 @@ static int derive_now(anni_adam *opt)
 	Flat f;
 
 	describe(opt, &f);
+	if (pv->fp8_twins && launch_fill_bytes(st, pv->d_wamax, 0,
+	    (size_t)opt->n_tensors * sizeof(uint32_t)) != 0)
+		return -1;
 	if (launch_derive(st, f) != 0)
 		return -1;
 	if (pv->fp8_twins) {
 		if (launch_amax_fold(st, f, nullptr) != 0)
 			return -1;
-		if (launch_fp8_twins(st, f, (uint8_t *)opt->d_param_fp8, opt->d_wscale,
-		    pv->d_wamax[pv->der_cur], pv->d_wamax[pv->der_cur ^ 1], opt->n_tensors,
-		    nullptr) != 0)
+		if (launch_fp8_twins(st, f, (uint8_t *)opt->d_param_fp8, opt->d_wscale, pv->d_wamax,
+		    opt->n_tensors, nullptr) != 0)
 			return -1;
-		pv->der_cur ^= 1;
 	}
 	return 0;
 }
@@ -591,7 +591,7 @@ static int enable_derived_body(anni_adam *opt, const anni_pack *packs, int n_pac
 	off_q = 0;
 	off_scale = round_up(fp8 ? (size_t)opt->n : 0, 256);
 	off_amax = off_scale + round_up((size_t)opt->n_tensors * sizeof(float), 256);
-	off_packs = off_amax + 2 * round_up((size_t)opt->n_tensors * sizeof(uint32_t), 256);
+	off_packs = off_amax + round_up((size_t)opt->n_tensors * sizeof(uint32_t), 256);
 	off_tamax = round_up(off_packs + (size_t)opt->n_tensors * sizeof(PackDesc), 256);
 	off_pack = round_up(off_tamax + (fp8 ? (size_t)((opt->n + kTile - 1) / kTile) * kWaves
 	    * sizeof(float) : 0), (size_t)2 << 20);
@@ -609,12 +609,9 @@ static int enable_derived_body(anni_adam *opt, const anni_pack *packs, int n_pac
 	base = (char *)pv->derived;
 	st = compute_stream();
 	ones.assign((size_t)opt->n_tensors, 1.0f);
-	pv->d_wamax[0] = (uint32_t *)(base + off_amax);
-	pv->d_wamax[1] = (uint32_t *)(base + off_amax
-	    + round_up((size_t)opt->n_tensors * sizeof(uint32_t), 256));
+	pv->d_wamax = (uint32_t *)(base + off_amax);
 	pv->d_packs = (PackDesc *)(base + off_packs);
 	pv->d_tile_amax = fp8 ? (float *)(base + off_tamax) : nullptr;
-	pv->der_cur = 0;
 	pv->fp8_twins = fp8 ? 1 : 0;
 	if (launch_fill_bytes(st, base, 0, total) != 0
 	    || !hip_ok(hipMemcpyAsync(base + off_scale, ones.data(),
@@ -679,7 +676,7 @@ static void describe(const anni_adam *opt, Flat *f)
 	f->tile_seg = pv->d_tile_seg;
 	f->gscale = opt->d_gscale;
 	if (pv->derived) {
-		f->der.wamax = pv->fp8_twins ? pv->d_wamax[pv->der_cur] : nullptr;
+		f->der.wamax = pv->fp8_twins ? pv->d_wamax : nullptr;
 		f->der.tile_amax = pv->d_tile_amax;
 		f->der.packs = pv->d_packs;
 		f->der.pack = (uint16_t *)opt->d_pack_bf16;
@@ -736,6 +733,14 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 	}
 	if (ev)
 		(void)hipEventRecord(ev[1], st);
+	/*
+	** The words the update raises start every step at zero, cleared on the stream by a fill
+	** kernel (not a memset node, and no state kept on the host: the step can be recorded into a
+	** graph and replayed).
+	*/
+	if (pv->fp8_twins && launch_fill_bytes(st, pv->d_wamax, 0,
+	    (size_t)opt->n_tensors * sizeof(uint32_t)) != 0)
+		return -1;
 	if (launch_update(st, f, c, grad_scale, norm) != 0)
 		return -1;
 	opt->t = t;
@@ -744,11 +749,9 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 	if (pv->fp8_twins) {
 		if (launch_amax_fold(st, f, norm.use_norm ? pv->d_state : nullptr) != 0)
 			return -1;
-		if (launch_fp8_twins(st, f, (uint8_t *)opt->d_param_fp8, opt->d_wscale,
-		    pv->d_wamax[pv->der_cur], pv->d_wamax[pv->der_cur ^ 1], opt->n_tensors,
-		    norm.use_norm ? pv->d_state : nullptr) != 0)
+		if (launch_fp8_twins(st, f, (uint8_t *)opt->d_param_fp8, opt->d_wscale, pv->d_wamax,
+		    opt->n_tensors, norm.use_norm ? pv->d_state : nullptr) != 0)
 			return -1;
-		pv->der_cur ^= 1;
 	}
 	if (ev)
 		(void)hipEventRecord(ev[3], st);

@@ -59,8 +59,8 @@ struct PackDesc {
 ** tensors flagged kSegFp8Twin: every wavefront leaves the maximum of its quarter of a whole tile
 ** in tile_amax[tile * kWaves + wave] (a plain store; tens of thousands of wavefronts raising
 ** one word per tensor were measured to cost the update 3-7 %), the few elements of tiles that
-** straddle tensors raise wamax[s] directly, and launch_amax_fold folds the tile maxima into
-** wamax.  A maximum does not depend on the order, so the result is deterministic.
+** straddle tensors raise wamax[s] directly (the caller clears wamax on the stream before
+** every launch_update / launch_derive), and launch_amax_fold folds the tile maxima into wamax.  A maximum does not depend on the order, so the result is deterministic.
 */
 struct Derived {
 	uint32_t	*wamax;
@@ -129,11 +129,11 @@ int	launch_derive(hipStream_t st, const Flat &f);
 int	launch_amax_fold(hipStream_t st, const Flat &f, const StepState *state);
 /*
 ** q = E4M3(p * (1 / scale_s)) for the tensors flagged kSegFp8Twin, scale_s from wamax[s]
-** (num/gpu_cuda.cu:826-851,927-938); wscale[s] receives the scale, wamax_next[0..n_tensors) is
-** cleared for the following step.  state (may be NULL): a skipped step leaves q and wscale alone.
+** (num/gpu_cuda.cu:826-851,927-938); wscale[s] receives the scale.  state (may be NULL): a
+** skipped step leaves q and wscale alone.
 */
 int	launch_fp8_twins(hipStream_t st, const Flat &f, uint8_t *q, float *wscale,
-		const uint32_t *wamax, uint32_t *wamax_next, int n_tensors, const StepState *state);
+		const uint32_t *wamax, int n_tensors, const StepState *state);
 int	launch_f32_to_bf16(hipStream_t st, uint16_t *dst, const float *src, int64_t n);
 /* pairs[2k] = m[first+k], pairs[2k+1] = v[first+k] as floats (bf16 moments widen exactly). */
 int	launch_mv_interleave(hipStream_t st, float *pairs, const void *m, const void *v,

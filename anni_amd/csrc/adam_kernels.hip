@@ -703,7 +703,6 @@ struct Fp8TwinArgs {
 	const Seg	*segs;
 	const int32_t	*tile_seg;
 	const uint32_t	*wamax;
-	uint32_t	*wamax_next;
 	float		*wscale;
 	int		n_tensors;
 	const StepState	*state;
@@ -727,7 +726,6 @@ __global__ __launch_bounds__(kThreads) void fp8_twin_kernel(Fp8TwinArgs a)
 		for (int s = tid; s < a.n_tensors; s += kThreads) {
 			if (!skipped && (a.segs[s].flags & kSegFp8Twin) != 0)
 				a.wscale[s] = scale_from_amax(__uint_as_float(a.wamax[s]));
-			a.wamax_next[s] = 0u;
 		}
 	}
 	if (skipped)
@@ -1154,11 +1152,11 @@ int launch_amax_fold(hipStream_t st, const Flat &f, const StepState *state)
 }
 
 int launch_fp8_twins(hipStream_t st, const Flat &f, uint8_t *q, float *wscale,
-	const uint32_t *wamax, uint32_t *wamax_next, int n_tensors, const StepState *state)
+	const uint32_t *wamax, int n_tensors, const StepState *state)
 {
 	Fp8TwinArgs a;
 
-	if (!f.p || f.n <= 0 || !f.segs || !f.tile_seg || !q || !wscale || !wamax || !wamax_next
+	if (!f.p || f.n <= 0 || !f.segs || !f.tile_seg || !q || !wscale || !wamax
 	    || n_tensors <= 0)
 		return -1;
 	a.p = f.p;
@@ -1167,7 +1165,6 @@ int launch_fp8_twins(hipStream_t st, const Flat &f, uint8_t *q, float *wscale,
 	a.segs = f.segs;
 	a.tile_seg = f.tile_seg;
 	a.wamax = wamax;
-	a.wamax_next = wamax_next;
 	a.wscale = wscale;
 	a.n_tensors = n_tensors;
 	a.state = state;
