@@ -185,7 +185,12 @@ double	anni_lr_step(double base_lr, int step);
 
 /* ---- stream plumbing ---------------------------------------------------- */
 
-/* The compute stream (a hipStream_t); anni_gpu_set_stream(NULL) restores the library's own. */
+/*
+** The compute stream (a hipStream_t); anni_gpu_set_stream(NULL) restores the library's own.
+** anni_adam_step_scaled on a stream under capture is recorded, not run (it allocates nothing and
+** waits for nothing); the recorded step keeps its lr, grad_scale, t and gradient flat.  Call
+** gpu_stream_sync before the capture begins so that no batched small copy is recorded with it.
+*/
 void	*anni_gpu_stream(void);
 void	anni_gpu_set_stream(void *hip_stream);
 
