@@ -38,26 +38,42 @@ __device__ __forceinline__ void st(T *p, T v)
 		*p = v;
 }
 
-/* Four consecutive values of a typed array, starting at element i (i % 4 == 0), as floats. */
+/* Four consecutive values of a typed array as they lie in memory (16, 8 or 4 bytes). */
+template <int T> struct RawQuad;
+template <> struct RawQuad<kF32> { f32x4 v; };
+template <> struct RawQuad<kBF16> { u32x2 v; };
+template <> struct RawQuad<kFP8> { uint32_t v; };
+
 template <int T, bool NT>
-__device__ __forceinline__ f32x4 load_quad(const void *base, int64_t i, float scale)
+__device__ __forceinline__ RawQuad<T> load_raw(const void *base, int64_t i)
+{
+	RawQuad<T> r;
+
+	if constexpr (T == kF32)
+		r.v = ld<NT>((const f32x4 *)((const float *)base + i));
+	else if constexpr (T == kBF16)
+		r.v = ld<NT>((const u32x2 *)((const uint16_t *)base + i));
+	else
+		r.v = ld<NT>((const uint32_t *)((const uint8_t *)base + i));
+	return r;
+}
+
+/* The four values as floats: bf16 widens exactly, E4M3 decodes exactly and is multiplied by scale. */
+template <int T>
+__device__ __forceinline__ f32x4 widen_raw(const RawQuad<T> &q, float scale)
 {
 	f32x4 r;
 
-	if (T == kF32) {
-		r = ld<NT>((const f32x4 *)((const float *)base + i));
-	} else if (T == kBF16) {
-		const u32x2 w = ld<NT>((const u32x2 *)((const uint16_t *)base + i));
-
-		r.x = __uint_as_float(w.x << 16);
-		r.y = __uint_as_float(w.x & 0xffff0000u);
-		r.z = __uint_as_float(w.y << 16);
-		r.w = __uint_as_float(w.y & 0xffff0000u);
+	if constexpr (T == kF32) {
+		r = q.v;
+	} else if constexpr (T == kBF16) {
+		r.x = __uint_as_float(q.v.x << 16);
+		r.y = __uint_as_float(q.v.x & 0xffff0000u);
+		r.z = __uint_as_float(q.v.y << 16);
+		r.w = __uint_as_float(q.v.y & 0xffff0000u);
 	} else {
-		const uint32_t w = ld<NT>((const uint32_t *)((const uint8_t *)base + i));
-
-		const f32x2_t lo = fp8_e4m3_decode2(w, false);
-		const f32x2_t hi = fp8_e4m3_decode2(w, true);
+		const f32x2_t lo = fp8_e4m3_decode2(q.v, false);
+		const f32x2_t hi = fp8_e4m3_decode2(q.v, true);
 
 		r.x = lo.x * scale;
 		r.y = lo.y * scale;
@@ -65,6 +81,13 @@ __device__ __forceinline__ f32x4 load_quad(const void *base, int64_t i, float sc
 		r.w = hi.y * scale;
 	}
 	return r;
+}
+
+/* Four consecutive values of a typed array, starting at element i (i % 4 == 0), as floats. */
+template <int T, bool NT>
+__device__ __forceinline__ f32x4 load_quad(const void *base, int64_t i, float scale)
+{
+	return widen_raw<T>(load_raw<T, NT>(base, i), scale);
 }
 
 /* Stores four floats into an f32 or bf16 array (bf16: round to nearest even). */
@@ -76,8 +99,8 @@ __device__ __forceinline__ void store_quad(void *base, int64_t i, f32x4 x)
 	} else {
 		u32x2 w;
 
-		w.x = bf16_rne(x.x) | (bf16_rne(x.y) << 16);
-		w.y = bf16_rne(x.z) | (bf16_rne(x.w) << 16);
+		w.x = bf16_rne2(x.x, x.y);
+		w.y = bf16_rne2(x.z, x.w);
 		st<NT>((u32x2 *)((uint16_t *)base + i), w);
 	}
 }
@@ -580,6 +603,226 @@ __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 	}
 }
 
+/* ---- the same update, software-pipelined (narrow storage modes) ----------------------- */
+
+/*
+** With bf16 moments or narrow gradients the update moves 22 - 28 bytes per element for the same
+** ~73 double-precision instructions, and the arithmetic shows: a wavefront that computes issues
+** no memory instruction for thousands of cycles, and with three wavefronts per SIMD the memory
+** pipeline runs dry whenever all of them compute (a kernel with the same nine streams and no
+** arithmetic is 9 % faster).  So here every wavefront has the loads of its NEXT tile in flight
+** while it computes the current one: two register stages, used in turn (the loop is unrolled by
+** two so that no stage is ever copied -- a copy would wait for the loads it copies).  A stage
+** holds the tile as it lies in memory (16 + 8 + 8 + 8 bytes per quad with bf16 storage) and is
+** widened quad by quad when it is consumed.  Arithmetic, rounding points and stores are those of
+** adam_update_kernel; results are bit-identical.
+*/
+template <int GT, int MT>
+struct Stage {
+	f32x4		P[kQuadsPerTile];
+	RawQuad<GT>	G[kQuadsPerTile];
+	RawQuad<MT>	M[kQuadsPerTile];
+	RawQuad<MT>	V[kQuadsPerTile];
+};
+
+struct TileInfo {
+	int64_t	base;
+	int64_t	end;
+	int	s;
+	bool	whole;
+	bool	vec;	/* a whole tile inside one tensor, not skipped: the staged path */
+};
+
+__device__ __forceinline__ TileInfo tile_info(const UpdateArgs &a, int64_t tile, bool skip)
+{
+	TileInfo t;
+
+	t.base = tile * kTile;
+	t.end = t.base + kTile < a.n ? t.base + kTile : a.n;
+	t.s = a.tile_seg ? a.tile_seg[tile] : 0;
+	t.whole = a.vec_ok && t.end - t.base == kTile;
+	t.vec = t.whole && !skip && (a.segs ? a.segs[t.s].end : a.n) >= t.end;
+	return t;
+}
+
+template <int GT, int MT, bool NT>
+__device__ __forceinline__ void stage_load(Stage<GT, MT> &st, const UpdateArgs &a, int64_t base,
+	int tid)
+{
+#pragma unroll
+	for (int u = 0; u < kQuadsPerTile; u++) {
+		const int64_t idx = base + (int64_t)(u * kThreads + tid) * kQuad;
+
+		st.G[u] = load_raw<GT, NT>(a.g, idx);
+		st.M[u] = load_raw<MT, NT>(a.m, idx);
+		st.V[u] = load_raw<MT, NT>(a.v, idx);
+		st.P[u] = ld<NT>((const f32x4 *)(a.p + idx));
+	}
+}
+
+template <int GT, int MT, bool NT, bool DER>
+__device__ __forceinline__ void stage_consume(const Stage<GT, MT> &st, const UpdateArgs &a,
+	int64_t tile, const TileInfo &t, double gs, int tid)
+{
+	const int s = t.s;
+	const uint32_t flags = a.segs ? a.segs[s].flags : a.uniform_flags;
+	const bool decay = a.c.decay_on && (flags & kSegDecay) != 0;
+	const bool twin = (flags & kSegTwin) != 0 && a.twin != nullptr;
+	const float sc = (GT == kFP8) ? a.gscale[s] : 1.0f;
+	const bool fp8w = DER && (flags & kSegFp8Twin) != 0 && a.der.wamax != nullptr;
+	const bool pk = DER && (flags & kSegPack) != 0 && a.der.pack != nullptr;
+	PackDesc pd = {0, 1u, 0u};
+	int64_t seg_begin = 0;
+	float amax_l = 0.0f;
+
+	if (pk) {
+		pd = a.der.packs[s];
+		seg_begin = a.segs[s].begin;
+	}
+#pragma unroll
+	for (int u = 0; u < kQuadsPerTile; u++) {
+		const int64_t idx = t.base + (int64_t)(u * kThreads + tid) * kQuad;
+		const f32x4 G = widen_raw<GT>(st.G[u], sc);
+		f32x4 M = widen_raw<MT>(st.M[u], 1.0f);
+		f32x4 V = widen_raw<MT>(st.V[u], 1.0f);
+		f32x4 P = st.P[u];
+
+#pragma unroll
+		for (int k = 0; k < kQuad; k++) {
+			const Elem e = adam_elem<(GT != kF32 || MT != kF32)>(P[k], G[k], M[k], V[k], gs, a.c,
+			    decay);
+
+			P[k] = e.p;
+			M[k] = e.m;
+			V[k] = e.v;
+		}
+		store_quad<kF32, NT>(a.p, idx, P);
+		store_quad<MT, NT>(a.m, idx, M);
+		store_quad<MT, NT>(a.v, idx, V);
+		zero_quad<GT, NT>(a.g, idx);
+		if (twin)
+			store_quad<kBF16, NT>(a.twin, idx, P);
+		if (fp8w)
+			amax_l = amax4(amax_l, P);
+		if (pk)
+			pack_quad<NT>(a.der.pack, pd, (uint32_t)(idx - seg_begin), P);
+	}
+	if (fp8w) {
+		amax_l = wave_max(amax_l);
+		if ((tid & 63) == 0)
+			a.der.tile_amax[tile * kWaves + (tid >> 6)] = amax_l;
+	}
+}
+
+/* A tile that is skipped, ragged or shared by several tensors: as in adam_update_kernel. */
+template <int GT, int MT, bool NT, bool DER>
+__device__ __forceinline__ void tile_slow(const UpdateArgs &a, const TileInfo &t, double gs,
+	bool skip, int tid)
+{
+	int s = t.s;
+
+	if (skip) {
+		if (t.whole) {
+#pragma unroll
+			for (int u = 0; u < kQuadsPerTile; u++)
+				zero_quad<GT, NT>(a.g, t.base + (int64_t)(u * kThreads + tid) * kQuad);
+		} else {
+			for (int64_t i = t.base + tid; i < t.end; i += kThreads)
+				zero_one<GT>(a.g, i);
+		}
+		return;
+	}
+	for (int64_t i = t.base + tid; i < t.end; i += kThreads) {
+		uint32_t flags = a.uniform_flags;
+		float sc = 1.0f;
+
+		if (a.segs) {
+			while (i >= a.segs[s].end)
+				s++;
+			flags = a.segs[s].flags;
+		}
+		if (GT == kFP8)
+			sc = a.gscale[s];
+		const Elem e = adam_elem<(GT != kF32 || MT != kF32)>(a.p[i], load_one<GT>(a.g, i, sc),
+		    load_one<MT>(a.m, i, 1.0f), load_one<MT>(a.v, i, 1.0f), gs, a.c,
+		    a.c.decay_on && (flags & kSegDecay) != 0);
+
+		a.p[i] = e.p;
+		store_one<MT>(a.m, i, e.m);
+		store_one<MT>(a.v, i, e.v);
+		zero_one<GT>(a.g, i);
+		if ((flags & kSegTwin) != 0 && a.twin != nullptr)
+			a.twin[i] = (uint16_t)bf16_rne(e.p);
+		if (DER && (flags & kSegFp8Twin) != 0 && a.der.wamax != nullptr) {
+			const float ab = fmaxf(0.0f, fabsf(e.p));
+
+			if (ab > 0.0f)
+				amax_raise(a.der.wamax + s, ab);
+		}
+		if (DER && (flags & kSegPack) != 0 && a.der.pack != nullptr)
+			pack_one(a.der.pack, a.der.packs[s], (uint32_t)(i - a.segs[s].begin), e.p);
+	}
+}
+
+template <int GT, int MT, bool NT, bool DER>
+__global__ __launch_bounds__(kThreads) void adam_update_pipe_kernel(UpdateArgs a)
+{
+	__shared__ double lds[4];
+	const int tid = threadIdx.x;
+	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
+	const int64_t step = gridDim.x;
+	double gs = a.grad_scale;
+	bool skip = false;
+	Stage<GT, MT> A, B;
+	TileInfo ta, tb;
+	int64_t tile = blockIdx.x;
+
+	if (a.use_norm) {
+		const double ss = partials_sum(a.partials, a.n_partials, lds);
+		const NormOut o = norm_decide(ss, a.clip, a.skip_nonfinite, gs, a.state,
+		    blockIdx.x == 0 && tid == 0);
+
+		gs = o.gs;
+		skip = o.skip;
+	}
+	if (tile >= n_tiles)
+		return;
+	ta = tile_info(a, tile, skip);
+	if (ta.vec)
+		stage_load<GT, MT, NT>(A, a, ta.base, tid);
+	for (;;) {
+		const int64_t t2 = tile + step;
+		const bool has_b = t2 < n_tiles;
+
+		if (has_b) {
+			tb = tile_info(a, t2, skip);
+			if (tb.vec)
+				stage_load<GT, MT, NT>(B, a, tb.base, tid);
+		}
+		if (ta.vec)
+			stage_consume<GT, MT, NT, DER>(A, a, tile, ta, gs, tid);
+		else
+			tile_slow<GT, MT, NT, DER>(a, ta, gs, skip, tid);
+		if (!has_b)
+			break;
+		const int64_t t3 = t2 + step;
+		const bool has_a = t3 < n_tiles;
+
+		if (has_a) {
+			ta = tile_info(a, t3, skip);
+			if (ta.vec)
+				stage_load<GT, MT, NT>(A, a, ta.base, tid);
+		}
+		if (tb.vec)
+			stage_consume<GT, MT, NT, DER>(B, a, t2, tb, gs, tid);
+		else
+			tile_slow<GT, MT, NT, DER>(a, tb, gs, skip, tid);
+		if (!has_a)
+			break;
+		tile = t3;
+	}
+}
+
 /* ---- derived outputs without an update, and the E4M3 twins ----------------------- */
 
 struct DeriveArgs {
@@ -1000,13 +1243,40 @@ int launch_finalize(hipStream_t st, const double *partials, int n_partials, doub
 #define ANNI_UPDATE_UNROLL_NARROW 4	/* bf16 moments / bf16 or fp8 gradients */
 #endif
 
+/* ANNI_PIPE=0 keeps the narrow storage modes on the plain kernel, 2 pipelines the all-f32 mode too (for comparison). */
+static int pipe_level(void)
+{
+	static int on = -1;
+
+	if (on < 0)
+		on = env_int("ANNI_PIPE", 1, 0, 2);
+	return on;
+}
+
 template <int GT, int MT>
 static void update_launch(hipStream_t st, int grid, const UpdateArgs &a)
 {
 	constexpr int U = (GT == kF32 && MT == kF32) ? ANNI_UPDATE_UNROLL : ANNI_UPDATE_UNROLL_NARROW;
-
+	constexpr bool narrow = GT != kF32 || MT != kF32;
 	const bool der = a.der.wamax != nullptr || a.der.pack != nullptr;
 
+	if (pipe_level() >= (narrow ? 1 : 2)) {
+		if (der) {
+			if (nt_on())
+				hipLaunchKernelGGL((adam_update_pipe_kernel<GT, MT, true, true>), dim3(grid),
+				    dim3(kThreads), 0, st, a);
+			else
+				hipLaunchKernelGGL((adam_update_pipe_kernel<GT, MT, false, true>), dim3(grid),
+				    dim3(kThreads), 0, st, a);
+		} else if (nt_on()) {
+			hipLaunchKernelGGL((adam_update_pipe_kernel<GT, MT, true, false>), dim3(grid),
+			    dim3(kThreads), 0, st, a);
+		} else {
+			hipLaunchKernelGGL((adam_update_pipe_kernel<GT, MT, false, false>), dim3(grid),
+			    dim3(kThreads), 0, st, a);
+		}
+		return;
+	}
 	if (der) {
 		if (nt_on())
 			hipLaunchKernelGGL((adam_update_kernel<GT, MT, U, true, true>), dim3(grid),

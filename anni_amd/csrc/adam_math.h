@@ -85,6 +85,20 @@ __device__ __forceinline__ uint32_t bf16_rne(float x)
 	return u >> 16;
 }
 
+/*
+** Two floats -> two bfloat16 in one word (x in the low half) with the gfx950 conversion
+** instruction: round to nearest even, NaN quieted; the same bits as bf16_rne for every float
+** (checked over all 2^32 patterns).
+*/
+typedef float f32x2_cv __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_cv __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t bf16_rne2(float x, float y)
+{
+	const f32x2_cv v = {x, y};
+
+	return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_cv));
+}
+
 __device__ __forceinline__ float bf16_widen(uint32_t h)
 {
 	return __uint_as_float(h << 16);

@@ -498,7 +498,9 @@ def main():
         "params_per_s": round(n / (ms_step * 1e-3), 1),
         "pct_of_hbm_peak": round(100.0 * step_gbps / HBM_PEAK_GBPS, 2),
         "event_ms_per_step": round(ev_ms / a.steps, 4),
-        "roofline": {"bound": "hbm", "kernel": "adam_update_kernel", "achieved": round(upd_gbps, 1),
+        "roofline": {"bound": "hbm",
+                     "kernel": "adam_update_kernel" if gt == 0 and mt == 0 else "adam_update_pipe_kernel",
+                     "achieved": round(upd_gbps, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(upd_gbps / HBM_PEAK_GBPS, 4),
                      "traffic": None if a.derived else TRAFFIC_BYTES.get(a.workload),

@@ -417,3 +417,22 @@ def test_fp8_quantizer_on_every_rounding_boundary(gpu, oracle):
     assert gpu.gpu_stream_sync() == 0
     want, scale = oracle.fp8_quantize(y)
     assert (q.download(np.uint8, y.size) == want).all() and sc.download(np.float32, 1)[0] == scale
+
+
+def test_bf16_conversion_on_all_float_patterns(gpu, oracle):
+    """The twins and bf16 moments are rounded by the gfx950 conversion instruction: all 2^32 float
+    bit patterns (every NaN, denormal and tie among them) give the bits of the oracle's
+    round-to-nearest-even routine, which is pinned against torch's bfloat16 cast."""
+    from anni_amd.lm_adam import DeviceBuffer
+    ch = 1 << 28
+    src, dst = DeviceBuffer(ch * 4), DeviceBuffer(ch * 2)
+    for c in range(16):
+        bits = np.arange(c * ch, (c + 1) * ch, dtype=np.uint64).astype(np.uint32)
+        x = bits.view(np.float32)
+        src.upload(x)
+        assert gpu.anni_f32_to_bf16(dst.ptr, src.ptr, ch) == 0
+        got = dst.download(np.uint16, ch)
+        bad = np.flatnonzero(got != oracle.bf16_rne(x))
+        assert bad.size == 0, [(hex(int(bits[i])), hex(int(got[i]))) for i in bad[:4]]
+    src.free()
+    dst.free()
