@@ -607,24 +607,19 @@ __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 
 /*
 ** With bf16 moments or narrow gradients the update moves 22 - 28 bytes per element for the same
-** ~73 double-precision instructions, and the arithmetic shows: a wavefront that computes issues
-** no memory instruction for thousands of cycles, and with three wavefronts per SIMD the memory
-** pipeline runs dry whenever all of them compute (a kernel with the same nine streams and no
-** arithmetic is 9 % faster).  So here every wavefront has the loads of its NEXT tile in flight
-** while it computes the current one: two register stages, used in turn (the loop is unrolled by
-** two so that no stage is ever copied -- a copy would wait for the loads it copies).  A stage
-** holds the tile as it lies in memory (16 + 8 + 8 + 8 bytes per quad with bf16 storage) and is
-** widened quad by quad when it is consumed.  Arithmetic, rounding points and stores are those of
-** adam_update_kernel; results are bit-identical.
+** arithmetic (~90 vector instructions per element, 55 of them double precision), and it shows: a
+** wavefront that computes issues no memory instruction for thousands of cycles, and the memory
+** pipeline runs dry whenever all wavefronts of a SIMD compute (a kernel with the same nine
+** streams and no arithmetic is 9 % faster).  So here every wavefront has the loads of its NEXT tile in flight
+** while it computes the current one: two register stages of half a tile each, used in turn
+** (never copied -- a copy would wait for the loads it copies): while the first half of a tile is
+** computed its second half is on the way, while the second half is computed the first half of
+** the wavefront's next tile.  A stage holds the data as they lie in memory (16 + 8 + 8 + 8 bytes
+** per quad with bf16 storage) and is widened quad by quad when it is consumed.  Half-tile stages
+** need ~110 registers (whole-tile stages ~150) and were measured 0.6 % faster with fp8 gradients.
+** Arithmetic, rounding points and stores are those of adam_update_kernel; results are
+** bit-identical.
 */
-template <int GT, int MT>
-struct Stage {
-	f32x4		P[kQuadsPerTile];
-	RawQuad<GT>	G[kQuadsPerTile];
-	RawQuad<MT>	M[kQuadsPerTile];
-	RawQuad<MT>	V[kQuadsPerTile];
-};
-
 struct TileInfo {
 	int64_t	base;
 	int64_t	end;
@@ -643,75 +638,6 @@ __device__ __forceinline__ TileInfo tile_info(const UpdateArgs &a, int64_t tile,
 	t.whole = a.vec_ok && t.end - t.base == kTile;
 	t.vec = t.whole && !skip && (a.segs ? a.segs[t.s].end : a.n) >= t.end;
 	return t;
-}
-
-template <int GT, int MT, bool NT>
-__device__ __forceinline__ void stage_load(Stage<GT, MT> &st, const UpdateArgs &a, int64_t base,
-	int tid)
-{
-#pragma unroll
-	for (int u = 0; u < kQuadsPerTile; u++) {
-		const int64_t idx = base + (int64_t)(u * kThreads + tid) * kQuad;
-
-		st.G[u] = load_raw<GT, NT>(a.g, idx);
-		st.M[u] = load_raw<MT, NT>(a.m, idx);
-		st.V[u] = load_raw<MT, NT>(a.v, idx);
-		st.P[u] = ld<NT>((const f32x4 *)(a.p + idx));
-	}
-}
-
-template <int GT, int MT, bool NT, bool DER>
-__device__ __forceinline__ void stage_consume(const Stage<GT, MT> &st, const UpdateArgs &a,
-	int64_t tile, const TileInfo &t, double gs, int tid)
-{
-	const int s = t.s;
-	const uint32_t flags = a.segs ? a.segs[s].flags : a.uniform_flags;
-	const bool decay = a.c.decay_on && (flags & kSegDecay) != 0;
-	const bool twin = (flags & kSegTwin) != 0 && a.twin != nullptr;
-	const float sc = (GT == kFP8) ? a.gscale[s] : 1.0f;
-	const bool fp8w = DER && (flags & kSegFp8Twin) != 0 && a.der.wamax != nullptr;
-	const bool pk = DER && (flags & kSegPack) != 0 && a.der.pack != nullptr;
-	PackDesc pd = {0, 1u, 0u};
-	int64_t seg_begin = 0;
-	float amax_l = 0.0f;
-
-	if (pk) {
-		pd = a.der.packs[s];
-		seg_begin = a.segs[s].begin;
-	}
-#pragma unroll
-	for (int u = 0; u < kQuadsPerTile; u++) {
-		const int64_t idx = t.base + (int64_t)(u * kThreads + tid) * kQuad;
-		const f32x4 G = widen_raw<GT>(st.G[u], sc);
-		f32x4 M = widen_raw<MT>(st.M[u], 1.0f);
-		f32x4 V = widen_raw<MT>(st.V[u], 1.0f);
-		f32x4 P = st.P[u];
-
-#pragma unroll
-		for (int k = 0; k < kQuad; k++) {
-			const Elem e = adam_elem<(GT != kF32 || MT != kF32)>(P[k], G[k], M[k], V[k], gs, a.c,
-			    decay);
-
-			P[k] = e.p;
-			M[k] = e.m;
-			V[k] = e.v;
-		}
-		store_quad<kF32, NT>(a.p, idx, P);
-		store_quad<MT, NT>(a.m, idx, M);
-		store_quad<MT, NT>(a.v, idx, V);
-		zero_quad<GT, NT>(a.g, idx);
-		if (twin)
-			store_quad<kBF16, NT>(a.twin, idx, P);
-		if (fp8w)
-			amax_l = amax4(amax_l, P);
-		if (pk)
-			pack_quad<NT>(a.der.pack, pd, (uint32_t)(idx - seg_begin), P);
-	}
-	if (fp8w) {
-		amax_l = wave_max(amax_l);
-		if ((tid & 63) == 0)
-			a.der.tile_amax[tile * kWaves + (tid >> 6)] = amax_l;
-	}
 }
 
 /* A tile that is skipped, ragged or shared by several tensors: as in adam_update_kernel. */
@@ -764,6 +690,77 @@ __device__ __forceinline__ void tile_slow(const UpdateArgs &a, const TileInfo &t
 	}
 }
 
+template <int GT, int MT>
+struct HalfStage {
+	f32x4		P[kQuadsPerTile / 2];
+	RawQuad<GT>	G[kQuadsPerTile / 2];
+	RawQuad<MT>	M[kQuadsPerTile / 2];
+	RawQuad<MT>	V[kQuadsPerTile / 2];
+};
+
+template <int GT, int MT, bool NT, int Q0>
+__device__ __forceinline__ void half_load(HalfStage<GT, MT> &st, const UpdateArgs &a, int64_t base,
+	int tid)
+{
+#pragma unroll
+	for (int u = 0; u < kQuadsPerTile / 2; u++) {
+		const int64_t idx = base + (int64_t)((Q0 + u) * kThreads + tid) * kQuad;
+
+		st.G[u] = load_raw<GT, NT>(a.g, idx);
+		st.M[u] = load_raw<MT, NT>(a.m, idx);
+		st.V[u] = load_raw<MT, NT>(a.v, idx);
+		st.P[u] = ld<NT>((const f32x4 *)(a.p + idx));
+	}
+}
+
+template <int GT, int MT, bool NT, bool DER, int Q0>
+__device__ __forceinline__ void half_consume(const HalfStage<GT, MT> &st, const UpdateArgs &a,
+	const TileInfo &t, double gs, int tid, float &amax_l)
+{
+	const int s = t.s;
+	const uint32_t flags = a.segs ? a.segs[s].flags : a.uniform_flags;
+	const bool decay = a.c.decay_on && (flags & kSegDecay) != 0;
+	const bool twin = (flags & kSegTwin) != 0 && a.twin != nullptr;
+	const float sc = (GT == kFP8) ? a.gscale[s] : 1.0f;
+	const bool fp8w = DER && (flags & kSegFp8Twin) != 0 && a.der.wamax != nullptr;
+	const bool pk = DER && (flags & kSegPack) != 0 && a.der.pack != nullptr;
+	PackDesc pd = {0, 1u, 0u};
+	int64_t seg_begin = 0;
+
+	if (pk) {
+		pd = a.der.packs[s];
+		seg_begin = a.segs[s].begin;
+	}
+#pragma unroll
+	for (int u = 0; u < kQuadsPerTile / 2; u++) {
+		const int64_t idx = t.base + (int64_t)((Q0 + u) * kThreads + tid) * kQuad;
+		const f32x4 G = widen_raw<GT>(st.G[u], sc);
+		f32x4 M = widen_raw<MT>(st.M[u], 1.0f);
+		f32x4 V = widen_raw<MT>(st.V[u], 1.0f);
+		f32x4 P = st.P[u];
+
+#pragma unroll
+		for (int k = 0; k < kQuad; k++) {
+			const Elem e = adam_elem<(GT != kF32 || MT != kF32)>(P[k], G[k], M[k], V[k], gs, a.c,
+			    decay);
+
+			P[k] = e.p;
+			M[k] = e.m;
+			V[k] = e.v;
+		}
+		store_quad<kF32, NT>(a.p, idx, P);
+		store_quad<MT, NT>(a.m, idx, M);
+		store_quad<MT, NT>(a.v, idx, V);
+		zero_quad<GT, NT>(a.g, idx);
+		if (twin)
+			store_quad<kBF16, NT>(a.twin, idx, P);
+		if (fp8w)
+			amax_l = amax4(amax_l, P);
+		if (pk)
+			pack_quad<NT>(a.der.pack, pd, (uint32_t)(idx - seg_begin), P);
+	}
+}
+
 template <int GT, int MT, bool NT, bool DER>
 __global__ __launch_bounds__(kThreads) void adam_update_pipe_kernel(UpdateArgs a)
 {
@@ -773,8 +770,8 @@ __global__ __launch_bounds__(kThreads) void adam_update_pipe_kernel(UpdateArgs a
 	const int64_t step = gridDim.x;
 	double gs = a.grad_scale;
 	bool skip = false;
-	Stage<GT, MT> A, B;
-	TileInfo ta, tb;
+	HalfStage<GT, MT> A, B;
+	TileInfo ta, tn;
 	int64_t tile = blockIdx.x;
 
 	if (a.use_norm) {
@@ -789,37 +786,36 @@ __global__ __launch_bounds__(kThreads) void adam_update_pipe_kernel(UpdateArgs a
 		return;
 	ta = tile_info(a, tile, skip);
 	if (ta.vec)
-		stage_load<GT, MT, NT>(A, a, ta.base, tid);
+		half_load<GT, MT, NT, 0>(A, a, ta.base, tid);
 	for (;;) {
-		const int64_t t2 = tile + step;
-		const bool has_b = t2 < n_tiles;
+		const int64_t next = tile + step;
+		const bool has = next < n_tiles;
+		float amax_l = 0.0f;
 
-		if (has_b) {
-			tb = tile_info(a, t2, skip);
-			if (tb.vec)
-				stage_load<GT, MT, NT>(B, a, tb.base, tid);
+		if (ta.vec) {
+			half_load<GT, MT, NT, kQuadsPerTile / 2>(B, a, ta.base, tid);
+			half_consume<GT, MT, NT, DER, 0>(A, a, ta, gs, tid, amax_l);
 		}
-		if (ta.vec)
-			stage_consume<GT, MT, NT, DER>(A, a, tile, ta, gs, tid);
-		else
+		if (has) {
+			tn = tile_info(a, next, skip);
+			if (tn.vec)
+				half_load<GT, MT, NT, 0>(A, a, tn.base, tid);
+		}
+		if (ta.vec) {
+			half_consume<GT, MT, NT, DER, kQuadsPerTile / 2>(B, a, ta, gs, tid, amax_l);
+			if (DER && a.der.wamax != nullptr && a.segs
+			    && (a.segs[ta.s].flags & kSegFp8Twin) != 0) {
+				amax_l = wave_max(amax_l);
+				if ((tid & 63) == 0)
+					a.der.tile_amax[tile * kWaves + (tid >> 6)] = amax_l;
+			}
+		} else {
 			tile_slow<GT, MT, NT, DER>(a, ta, gs, skip, tid);
-		if (!has_b)
-			break;
-		const int64_t t3 = t2 + step;
-		const bool has_a = t3 < n_tiles;
-
-		if (has_a) {
-			ta = tile_info(a, t3, skip);
-			if (ta.vec)
-				stage_load<GT, MT, NT>(A, a, ta.base, tid);
 		}
-		if (tb.vec)
-			stage_consume<GT, MT, NT, DER>(B, a, t2, tb, gs, tid);
-		else
-			tile_slow<GT, MT, NT, DER>(a, tb, gs, skip, tid);
-		if (!has_a)
+		if (!has)
 			break;
-		tile = t3;
+		tile = next;
+		ta = tn;
 	}
 }
 
