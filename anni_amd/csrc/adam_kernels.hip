@@ -294,8 +294,13 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(SumsqArgs a)
 	for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
 		const int64_t base = tile * kTile;
 		const int64_t end = base + kTile < a.n ? base + kTile : a.n;
-		int s = a.tile_seg ? a.tile_seg[tile] : 0;
-		const int64_t seg_end = a.segs ? a.segs[s].end : a.n;
+		/*
+		** Only fp8 gradients carry a scale per tensor; for the others the sum does not care
+		** where tensors begin, and two dependent scalar loads per tile ahead of the vector
+		** loads cost 8 % of the kernel.
+		*/
+		int s = (GT == kFP8 && a.tile_seg) ? a.tile_seg[tile] : 0;
+		const int64_t seg_end = (GT == kFP8 && a.segs) ? a.segs[s].end : a.n;
 
 		if (a.vec_ok && end - base == kTile && seg_end >= end) {
 			const float sc = (GT == kFP8) ? a.gscale[s] : 1.0f;
@@ -320,11 +325,12 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(SumsqArgs a)
 			for (int64_t i = base + tid; i < end; i += kThreads) {
 				float sc = 1.0f;
 
-				if (a.segs)
-					while (i >= a.segs[s].end)
-						s++;
-				if (GT == kFP8)
+				if (GT == kFP8) {
+					if (a.segs)
+						while (i >= a.segs[s].end)
+							s++;
 					sc = a.gscale[s];
+				}
 				const double x = (double)load_one<GT>(a.g, i, sc) * a.grad_scale;
 
 				acc0 += x * x;
@@ -465,6 +471,36 @@ struct UpdateArgs {
 };
 
 /*
+** What a workgroup needs to know about a tile before it can issue the tile's loads: a chain of
+** dependent scalar loads (tile -> tensor -> end, flags, scale).  The kernels look it up one tile
+** ahead, so the chain runs while the current tile is computed.
+*/
+struct TileInfo {
+	int64_t		base;
+	int64_t		end;
+	int		s;
+	uint32_t	flags;
+	float		sc;	/* fp8 gradients: the tensor's scale */
+	bool		whole;
+	bool		vec;	/* a whole tile inside one tensor, not skipped: the vector path */
+};
+
+template <int GT>
+__device__ __forceinline__ TileInfo tile_info(const UpdateArgs &a, int64_t tile, bool skip)
+{
+	TileInfo t;
+
+	t.base = tile * kTile;
+	t.end = t.base + kTile < a.n ? t.base + kTile : a.n;
+	t.s = a.tile_seg ? a.tile_seg[tile] : 0;
+	t.flags = a.segs ? a.segs[t.s].flags : a.uniform_flags;
+	t.sc = (GT == kFP8) ? a.gscale[t.s] : 1.0f;
+	t.whole = a.vec_ok && t.end - t.base == kTile;
+	t.vec = t.whole && !skip && (a.segs ? a.segs[t.s].end : a.n) >= t.end;
+	return t;
+}
+
+/*
 ** U = quads a lane keeps in flight at once (kQuadsPerTile % U == 0).  With narrow storage
 ** types the kernel moves fewer bytes per element for the same arithmetic, so those modes
 ** take the cheaper constant division (adam_math.h) and the deeper unroll.
@@ -490,13 +526,20 @@ __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 		gs = o.gs;
 		skip = o.skip;
 	}
-	for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-		const int64_t base = tile * kTile;
-		const int64_t end = base + kTile < a.n ? base + kTile : a.n;
-		int s = a.tile_seg ? a.tile_seg[tile] : 0;
-		const int64_t seg_end = a.segs ? a.segs[s].end : a.n;
-		const bool whole = a.vec_ok && end - base == kTile;
+	TileInfo cur = tile_info<GT>(a, blockIdx.x < n_tiles ? (int64_t)blockIdx.x : 0, skip);
 
+	for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+		const int64_t ahead = tile + gridDim.x < n_tiles ? tile + gridDim.x : tile;
+		const TileInfo nxt = tile_info<GT>(a, ahead, skip);	/* used after this tile */
+		const int64_t base = cur.base;
+		const int64_t end = cur.end;
+		int s = cur.s;
+		const bool whole = cur.whole;
+		const bool vec = cur.vec;
+		const uint32_t flags = cur.flags;
+		const float sc = cur.sc;
+
+		cur = nxt;
 		if (skip) {
 			/* Non-finite norm: p, m, v and the twins stay as they are; gradients are cleared. */
 			if (whole) {
@@ -509,11 +552,9 @@ __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 			}
 			continue;
 		}
-		if (whole && seg_end >= end) {
-			const uint32_t flags = a.segs ? a.segs[s].flags : a.uniform_flags;
+		if (vec) {
 			const bool decay = a.c.decay_on && (flags & kSegDecay) != 0;
 			const bool twin = (flags & kSegTwin) != 0 && a.twin != nullptr;
-			const float sc = (GT == kFP8) ? a.gscale[s] : 1.0f;
 			const bool fp8w = DER && (flags & kSegFp8Twin) != 0 && a.der.wamax != nullptr;
 			const bool pk = DER && (flags & kSegPack) != 0 && a.der.pack != nullptr;
 			PackDesc pd = {0, 1u, 0u};
@@ -620,26 +661,6 @@ __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 ** Arithmetic, rounding points and stores are those of adam_update_kernel; results are
 ** bit-identical.
 */
-struct TileInfo {
-	int64_t	base;
-	int64_t	end;
-	int	s;
-	bool	whole;
-	bool	vec;	/* a whole tile inside one tensor, not skipped: the staged path */
-};
-
-__device__ __forceinline__ TileInfo tile_info(const UpdateArgs &a, int64_t tile, bool skip)
-{
-	TileInfo t;
-
-	t.base = tile * kTile;
-	t.end = t.base + kTile < a.n ? t.base + kTile : a.n;
-	t.s = a.tile_seg ? a.tile_seg[tile] : 0;
-	t.whole = a.vec_ok && t.end - t.base == kTile;
-	t.vec = t.whole && !skip && (a.segs ? a.segs[t.s].end : a.n) >= t.end;
-	return t;
-}
-
 /* A tile that is skipped, ragged or shared by several tensors: as in adam_update_kernel. */
 template <int GT, int MT, bool NT, bool DER>
 __device__ __forceinline__ void tile_slow(const UpdateArgs &a, const TileInfo &t, double gs,
@@ -718,10 +739,10 @@ __device__ __forceinline__ void half_consume(const HalfStage<GT, MT> &st, const 
 	const TileInfo &t, double gs, int tid, float &amax_l)
 {
 	const int s = t.s;
-	const uint32_t flags = a.segs ? a.segs[s].flags : a.uniform_flags;
+	const uint32_t flags = t.flags;
 	const bool decay = a.c.decay_on && (flags & kSegDecay) != 0;
 	const bool twin = (flags & kSegTwin) != 0 && a.twin != nullptr;
-	const float sc = (GT == kFP8) ? a.gscale[s] : 1.0f;
+	const float sc = t.sc;
 	const bool fp8w = DER && (flags & kSegFp8Twin) != 0 && a.der.wamax != nullptr;
 	const bool pk = DER && (flags & kSegPack) != 0 && a.der.pack != nullptr;
 	PackDesc pd = {0, 1u, 0u};
@@ -784,7 +805,7 @@ __global__ __launch_bounds__(kThreads) void adam_update_pipe_kernel(UpdateArgs a
 	}
 	if (tile >= n_tiles)
 		return;
-	ta = tile_info(a, tile, skip);
+	ta = tile_info<GT>(a, tile, skip);
 	if (ta.vec)
 		half_load<GT, MT, NT, 0>(A, a, ta.base, tid);
 	for (;;) {
@@ -797,14 +818,13 @@ __global__ __launch_bounds__(kThreads) void adam_update_pipe_kernel(UpdateArgs a
 			half_consume<GT, MT, NT, DER, 0>(A, a, ta, gs, tid, amax_l);
 		}
 		if (has) {
-			tn = tile_info(a, next, skip);
+			tn = tile_info<GT>(a, next, skip);
 			if (tn.vec)
 				half_load<GT, MT, NT, 0>(A, a, tn.base, tid);
 		}
 		if (ta.vec) {
 			half_consume<GT, MT, NT, DER, kQuadsPerTile / 2>(B, a, ta, gs, tid, amax_l);
-			if (DER && a.der.wamax != nullptr && a.segs
-			    && (a.segs[ta.s].flags & kSegFp8Twin) != 0) {
+			if (DER && a.der.wamax != nullptr && (ta.flags & kSegFp8Twin) != 0) {
 				amax_l = wave_max(amax_l);
 				if ((tid & 63) == 0)
 					a.der.tile_amax[tile * kWaves + (tid >> 6)] = amax_l;
