@@ -39,7 +39,7 @@ WORKLOADS = {
 ELEM = {0: 4, 1: 2, 2: 1}
 # HBM bytes per launch of the update kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled
 # by what the counter reads for a plain copy kernel of known size (summaries under profiles/).
-TRAFFIC_BYTES = {"555m": 18902963578, "185m": 5711519396, "555m-bf16": 12232667785,
+TRAFFIC_BYTES = {"555m": 18902966198, "185m": 5711517786, "555m-bf16": 12232667785,
                  "1p4b-fp8": 39589398592}
 STORAGE = {"185m": "f32 p/g/m/v + bf16 twin", "555m": "f32 p/g/m/v + bf16 twin",
            "555m-bf16": "f32 p, bf16 g/m/v + bf16 twin",
