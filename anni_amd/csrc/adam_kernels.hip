@@ -360,36 +360,31 @@ __global__ __launch_bounds__(kThreads) void sumsq_fp8_kernel(SumsqArgs a)
 
 	for (int64_t t0 = blockIdx.x; t0 < n_tiles; t0 += (int64_t)gridDim.x * kAhead) {
 		u32x4 W[kAhead];
-		double s2[kAhead];
-		bool fast[kAhead];
+		bool whole[kAhead];
 
+		/* the loads of whole tiles go out first: they do not depend on the tensor table */
 #pragma unroll
 		for (int j = 0; j < kAhead; j++) {
 			const int64_t tile = t0 + (int64_t)j * gridDim.x;
 
-			fast[j] = false;
-			s2[j] = 0.0;
+			whole[j] = a.vec_ok && tile < n_tiles && (tile + 1) * kTile <= a.n;
 			W[j] = u32x4{0u, 0u, 0u, 0u};
-			if (tile < n_tiles) {
-				const int64_t base = tile * kTile;
-				const int64_t end = base + kTile < a.n ? base + kTile : a.n;
-				const int s = a.tile_seg ? a.tile_seg[tile] : 0;
-				const int64_t seg_end = a.segs ? a.segs[s].end : a.n;
-
-				if (a.vec_ok && end - base == kTile && seg_end >= end) {
-					const double sc = (double)a.gscale[s] * a.grad_scale;
-
-					fast[j] = true;
-					s2[j] = sc * sc;
-					W[j] = ld<NT>((const u32x4 *)((const uint8_t *)a.g + base) + tid);
-				}
-			}
+			if (whole[j])
+				W[j] = ld<NT>((const u32x4 *)((const uint8_t *)a.g + tile * kTile) + tid);
 		}
 #pragma unroll
 		for (int j = 0; j < kAhead; j++) {
 			const int64_t tile = t0 + (int64_t)j * gridDim.x;
 
-			if (fast[j]) {
+			if (tile >= n_tiles)
+				continue;
+			const int64_t base = tile * kTile;
+			const int64_t end = base + kTile < a.n ? base + kTile : a.n;
+			int s = a.tile_seg ? a.tile_seg[tile] : 0;
+			const int64_t seg_end = a.segs ? a.segs[s].end : a.n;
+
+			if (whole[j] && seg_end >= end) {
+				const double sc = (double)a.gscale[s] * a.grad_scale;
 				double t = 0.0;
 
 #pragma unroll
@@ -402,12 +397,8 @@ __global__ __launch_bounds__(kThreads) void sumsq_fp8_kernel(SumsqArgs a)
 					t += (double)(hi.x * hi.x);
 					t += (double)(hi.y * hi.y);
 				}
-				acc += s2[j] * t;
-			} else if (tile < n_tiles) {
-				const int64_t base = tile * kTile;
-				const int64_t end = base + kTile < a.n ? base + kTile : a.n;
-				int s = a.tile_seg ? a.tile_seg[tile] : 0;
-
+				acc += (sc * sc) * t;
+			} else {
 				for (int64_t i = base + tid; i < end; i += kThreads) {
 					if (a.segs)
 						while (i >= a.segs[s].end)
