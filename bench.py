@@ -47,8 +47,9 @@ STORAGE = {"185m": "f32 p/g/m/v + bf16 twin", "555m": "f32 p/g/m/v + bf16 twin",
            "1p4b": "f32 p/g/m/v + bf16 twin"}
 
 
-def fill_grad_slots(L, opt, tensors, count, grad_type, seed):
-    """Fills the arena's `count` gradient slots, each ~N(0, 1e-3) in the workload's storage type.
+def fill_grad_slots(L, opt, tensors, count, grad_type, seed, first_step=0):
+    """Fills the arena's first `count` gradient slots for the steps first_step .. first_step + count - 1,
+    each ~N(0, 1e-3) in the workload's storage type (a fresh random stream per step).
     Returns the slot pointers and, for fp8, one per-tensor scale array per slot."""
     from anni_amd.lm_adam import DeviceBuffer
     n = opt.n
@@ -58,7 +59,7 @@ def fill_grad_slots(L, opt, tensors, count, grad_type, seed):
         slot = opt.grad_slot(k)
         assert slot
         dst = slot if grad_type == 0 else stage.ptr
-        assert L.anni_fill_normal_f32(dst, n, seed, 1000 + k, 0.0, 1e-3) == 0
+        assert L.anni_fill_normal_f32(dst, n, seed, 1000 + first_step + k, 0.0, 1e-3) == 0
         sc = None
         if grad_type == 1:
             assert L.anni_f32_to_bf16(slot, stage.ptr, n) == 0
@@ -409,15 +410,21 @@ def main():
                 packs.append((names.index("blk%d.%s" % (b, w)), d, pack_elems + k * d, 3 * d))
             pack_elems += 3 * d * d
     total = a.steps + a.warmup
+    # Gradient slots: one per step while they fit two 16 GiB regions of device memory (13 at 555M);
+    # beyond that the steps run in batches, the slots being refilled between batches with the
+    # clock stopped, so that any --steps keeps the arena, and with it the placement, the same.
+    n_params = sum(t[1] for t in tensors)
+    slot_bytes = -(-n_params * ELEM[gt] // (2 << 20)) * (2 << 20)
+    n_slots = min(total, max(4, (32 << 30) // slot_bytes))
     opt = LmAdam(tensors, grad_type=gt, moment_type=mt, twins=True, skip_nonfinite=True,
-                 grad_slots=total, layout={"auto": 0, "compact": 1, "spread": 2}[a.layout],
+                 grad_slots=n_slots, layout={"auto": 0, "compact": 1, "spread": 2}[a.layout],
                  beta2=0.95, weight_decay=0.1, grad_clip=1.0)
     n = opt.n
     assert L.anni_fill_normal_f32(opt.o.d_param, n, 20260101, 1, 0.0, 0.02) == 0
     if a.derived:
         opt.enable_derived(packs, pack_elems)
     opt.seed_twins()
-    ring, scales = fill_grad_slots(L, opt, tensors, total, gt, 20260101)
+    ring, scales = fill_grad_slots(L, opt, tensors, min(n_slots, total), gt, 20260101)
 
     # per-step inputs: warmup(100)+cosine lr at schedule steps 0.., grad scale straddling the clip
     from anni_amd import lm_adam
@@ -425,10 +432,10 @@ def main():
     unit = 1.0 / (math.sqrt(n) * 1e-3)
     gss = [unit * (1.7 if s % 2 else 0.6) for s in range(total)]
 
-    per_step_ms, skipped_steps = [], []
+    per_step_ms, skipped_steps, der_acc = [], [], [0.0]
 
     def run(first, count, per_kernel):
-        ptrs = (C.c_void_p * count)(*[ring[first + i] for i in range(count)])
+        ptrs = (C.c_void_p * count)(*[ring[(first + i) % n_slots] for i in range(count)])
         lr = (C.c_double * count)(*lrs[first:first + count])
         gs = (C.c_double * count)(*gss[first:first + count])
         ms, ms_a, ms_b = C.c_float(0), C.c_float(0), C.c_float(0)
@@ -438,7 +445,7 @@ def main():
             tot = sa = sb = 0.0
             for i in range(count):
                 if gt == 2:
-                    opt.o.d_gscale = scales[first + i].ptr
+                    opt.o.d_gscale = scales[(first + i) % n_slots].ptr
                 one = (C.c_void_p * 1)(ptrs[i])
                 rc = L.anni_adam_time_steps(opt.h, 1, one, 1, C.byref(C.c_double(lr[i])),
                                             C.byref(C.c_double(gs[i])), C.byref(ms),
@@ -448,6 +455,7 @@ def main():
                 tot, sa, sb = tot + ms.value, sa + ms_a.value, sb + ms_b.value
                 if per_kernel:
                     per_step_ms.append(ms.value)
+                    der_acc[0] += L.anni_adam_timed_derived_ms(opt.h) if a.derived else 0.0
                     o = opt.sync_stats() if a.ref_jsonl else None
                     if o is not None and (o.last_skipped or not math.isfinite(o.last_grad_norm)):
                         skipped_steps.append(first + i)
@@ -456,15 +464,31 @@ def main():
                                     C.byref(ms_a) if per_kernel else None,
                                     C.byref(ms_b) if per_kernel else None)
         assert rc == 0, L.gpu_debug_last_error()
+        if per_kernel and a.derived:
+            der_acc[0] += L.anni_adam_timed_derived_ms(opt.h)
         return ms.value, ms_a.value, ms_b.value
 
-    if a.warmup:
-        run(0, a.warmup, False)
-    L.gpu_device_sync()
-    t0 = time.perf_counter()
-    ev_ms, ms_sumsq, ms_update = run(a.warmup, a.steps, True)
-    L.gpu_device_sync()
-    wall_ms = (time.perf_counter() - t0) * 1e3
+    # steps 0 .. total-1 in batches of n_slots (one batch when they all fit); the clock runs only
+    # over the timed steps of each batch, bracketed by device synchronisations
+    ev_ms = ms_sumsq = ms_update = wall_ms = 0.0
+    for b0 in range(0, total, n_slots):
+        b1 = min(b0 + n_slots, total)
+        if b0:
+            refill = fill_grad_slots(L, opt, tensors, b1 - b0, gt, 20260101, b0)
+            for sc_old in scales:
+                if sc_old is not None:
+                    sc_old.free()
+            ring, scales = refill
+        w1 = min(max(a.warmup, b0), b1)                 # [b0, w1) untimed, [w1, b1) timed
+        if w1 > b0:
+            run(b0, w1 - b0, False)
+        if b1 > w1:
+            L.gpu_device_sync()
+            t0 = time.perf_counter()
+            e, sa, sb = run(w1, b1 - w1, True)
+            L.gpu_device_sync()
+            wall_ms += (time.perf_counter() - t0) * 1e3
+            ev_ms, ms_sumsq, ms_update = ev_ms + e, ms_sumsq + sa, ms_update + sb
 
     peak_mb = 0.0
     fr, tt = C.c_size_t(0), C.c_size_t(0)
@@ -511,7 +535,7 @@ def main():
         "last_grad_norm": st.last_grad_norm, "last_clipped": int(st.last_clipped),
     }
     if a.derived:
-        der_ms = L.anni_adam_timed_derived_ms(opt.h) / a.steps
+        der_ms = der_acc[0] / a.steps
         out["config"]["derived"] = {"both": "E4M3 twins of every matrix + packed [Wq|Wk|Wv] per block",
                                     "fp8": "E4M3 twins of every matrix",
                                     "pack": "packed [Wq|Wk|Wv] per block"}[a.derived]
