@@ -281,17 +281,17 @@ struct SumsqArgs {
 	double		grad_scale;
 	double		*partials;
 	int		vec_ok;
+	int64_t		keep_from;	/* tiles from here on are read with ordinary (cacheable) loads */
 };
 
+/* The tiles first, first + step, ... below `stop`, added to the lane's four running sums. */
 template <int GT, bool NT>
-__global__ __launch_bounds__(kThreads) void sumsq_kernel(SumsqArgs a)
+__device__ __forceinline__ int64_t sumsq_tiles(const SumsqArgs &a, int64_t first, int64_t step,
+	int64_t stop, int tid, double (&acc)[4])
 {
-	__shared__ double lds[4];
-	const int tid = threadIdx.x;
-	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
-	double acc0 = 0.0, acc1 = 0.0, acc2 = 0.0, acc3 = 0.0;
+	int64_t tile = first;
 
-	for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+	for (; tile < stop; tile += step) {
 		const int64_t base = tile * kTile;
 		const int64_t end = base + kTile < a.n ? base + kTile : a.n;
 		/*
@@ -316,10 +316,10 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(SumsqArgs a)
 				const double x2 = (double)G[u].z * a.grad_scale;
 				const double x3 = (double)G[u].w * a.grad_scale;
 
-				acc0 += x0 * x0;
-				acc1 += x1 * x1;
-				acc2 += x2 * x2;
-				acc3 += x3 * x3;
+				acc[0] += x0 * x0;
+				acc[1] += x1 * x1;
+				acc[2] += x2 * x2;
+				acc[3] += x3 * x3;
 			}
 		} else {
 			for (int64_t i = base + tid; i < end; i += kThreads) {
@@ -333,11 +333,31 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(SumsqArgs a)
 				}
 				const double x = (double)load_one<GT>(a.g, i, sc) * a.grad_scale;
 
-				acc0 += x * x;
+				acc[0] += x * x;
 			}
 		}
 	}
-	const double total = block_sum((acc0 + acc1) + (acc2 + acc3), lds);
+	return tile;
+}
+
+/*
+** A workgroup takes the tiles blockIdx.x, blockIdx.x + gridDim.x, ... in rising order.  The
+** tiles from `keep_from` on are read with ordinary loads, so the memory-side cache keeps them for
+** the update kernel that follows; the others stream past it.
+*/
+template <int GT, bool NT>
+__global__ __launch_bounds__(kThreads) void sumsq_kernel(SumsqArgs a)
+{
+	__shared__ double lds[4];
+	const int tid = threadIdx.x;
+	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
+	const int64_t keep_from = NT ? (a.keep_from < n_tiles ? a.keep_from : n_tiles) : 0;
+	double acc[4] = {0.0, 0.0, 0.0, 0.0};
+	int64_t tile;
+
+	tile = sumsq_tiles<GT, NT>(a, blockIdx.x, gridDim.x, keep_from, tid, acc);
+	(void)sumsq_tiles<GT, false>(a, tile, gridDim.x, n_tiles, tid, acc);
+	const double total = block_sum((acc[0] + acc[1]) + (acc[2] + acc[3]), lds);
 
 	if (tid == 0)
 		a.partials[blockIdx.x] = total;
@@ -348,24 +368,24 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(SumsqArgs a)
 ** of an E4M3 value is exact in float and the inner sums are exact in double, so only the
 ** per-tile products round.  One 16-byte load (16 codes) per lane per tile, four tiles in flight.
 */
+constexpr int kSumsqFp8Ahead = 4;
+
+/* The groups of kAhead tiles t0, t0 + step, ... that begin below `stop`; returns the next t0. */
 template <bool NT>
-__global__ __launch_bounds__(kThreads) void sumsq_fp8_kernel(SumsqArgs a)
+__device__ __forceinline__ int64_t sumsq_fp8_tiles(const SumsqArgs &a, int64_t t0, int64_t step,
+	int64_t stop, int64_t n_tiles, int tid, double &acc)
 {
 	typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-	__shared__ double lds[4];
-	constexpr int kAhead = 4;
-	const int tid = threadIdx.x;
-	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
-	double acc = 0.0;
+	constexpr int kAhead = kSumsqFp8Ahead;
 
-	for (int64_t t0 = blockIdx.x; t0 < n_tiles; t0 += (int64_t)gridDim.x * kAhead) {
+	for (; t0 < stop; t0 += step * kAhead) {
 		u32x4 W[kAhead];
 		bool whole[kAhead];
 
 		/* the loads of whole tiles go out first: they do not depend on the tensor table */
 #pragma unroll
 		for (int j = 0; j < kAhead; j++) {
-			const int64_t tile = t0 + (int64_t)j * gridDim.x;
+			const int64_t tile = t0 + (int64_t)j * step;
 
 			whole[j] = a.vec_ok && tile < n_tiles && (tile + 1) * kTile <= a.n;
 			W[j] = u32x4{0u, 0u, 0u, 0u};
@@ -374,7 +394,7 @@ __global__ __launch_bounds__(kThreads) void sumsq_fp8_kernel(SumsqArgs a)
 		}
 #pragma unroll
 		for (int j = 0; j < kAhead; j++) {
-			const int64_t tile = t0 + (int64_t)j * gridDim.x;
+			const int64_t tile = t0 + (int64_t)j * step;
 
 			if (tile >= n_tiles)
 				continue;
@@ -411,6 +431,25 @@ __global__ __launch_bounds__(kThreads) void sumsq_fp8_kernel(SumsqArgs a)
 			}
 		}
 	}
+	return t0;
+}
+
+/*
+** A workgroup takes its tiles in groups of kSumsqFp8Ahead, one grid width apart; keep_from is a
+** whole number of such rounds of the grid, so every workgroup changes over between two groups.
+*/
+template <bool NT>
+__global__ __launch_bounds__(kThreads) void sumsq_fp8_kernel(SumsqArgs a)
+{
+	__shared__ double lds[4];
+	const int tid = threadIdx.x;
+	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
+	const int64_t keep_from = NT ? (a.keep_from < n_tiles ? a.keep_from : n_tiles) : 0;
+	double acc = 0.0;
+	int64_t t0;
+
+	t0 = sumsq_fp8_tiles<NT>(a, blockIdx.x, gridDim.x, keep_from, n_tiles, tid, acc);
+	(void)sumsq_fp8_tiles<false>(a, t0, gridDim.x, n_tiles, n_tiles, tid, acc);
 	const double total = block_sum(acc, lds);
 
 	if (tid == 0)
@@ -449,6 +488,7 @@ struct UpdateArgs {
 	const float	*gscale;
 	uint32_t	uniform_flags;
 	int		vec_ok;
+	int		reverse;	/* walk the tiles from the last to the first */
 	StepConsts	c;
 	double		grad_scale;
 	/* norm */
@@ -467,6 +507,7 @@ struct UpdateArgs {
 ** ahead, so the chain runs while the current tile is computed.
 */
 struct TileInfo {
+	int64_t		tile;	/* the tile's place in the flat */
 	int64_t		base;
 	int64_t		end;
 	int		s;
@@ -477,10 +518,12 @@ struct TileInfo {
 };
 
 template <int GT>
-__device__ __forceinline__ TileInfo tile_info(const UpdateArgs &a, int64_t tile, bool skip)
+__device__ __forceinline__ TileInfo tile_info(const UpdateArgs &a, int64_t turn, bool skip)
 {
 	TileInfo t;
+	const int64_t tile = a.reverse ? (a.n + kTile - 1) / kTile - 1 - turn : turn;
 
+	t.tile = tile;
 	t.base = tile * kTile;
 	t.end = t.base + kTile < a.n ? t.base + kTile : a.n;
 	t.s = a.tile_seg ? a.tile_seg[tile] : 0;
@@ -529,6 +572,7 @@ __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 		const bool vec = cur.vec;
 		const uint32_t flags = cur.flags;
 		const float sc = cur.sc;
+		const int64_t place = cur.tile;
 
 		cur = nxt;
 		if (skip) {
@@ -598,7 +642,7 @@ __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 			if (fp8w) {
 				amax_l = wave_max(amax_l);
 				if ((tid & 63) == 0)
-					a.der.tile_amax[tile * kWaves + (tid >> 6)] = amax_l;
+					a.der.tile_amax[place * kWaves + (tid >> 6)] = amax_l;
 			}
 		} else {
 			for (int64_t i = base + tid; i < end; i += kThreads) {
@@ -818,7 +862,7 @@ __global__ __launch_bounds__(kThreads) void adam_update_pipe_kernel(UpdateArgs a
 			if (DER && a.der.wamax != nullptr && (ta.flags & kSegFp8Twin) != 0) {
 				amax_l = wave_max(amax_l);
 				if ((tid & 63) == 0)
-					a.der.tile_amax[tile * kWaves + (tid >> 6)] = amax_l;
+					a.der.tile_amax[ta.tile * kWaves + (tid >> 6)] = amax_l;
 			}
 		} else {
 			tile_slow<GT, MT, NT, DER>(a, ta, gs, skip, tid);
@@ -1157,6 +1201,26 @@ static bool nt_on(void)
 	return on != 0;
 }
 
+/* ANNI_REVERSE=0: the update walks the tiles from the first to the last. */
+static bool reverse_on(void)
+{
+	static int on = -1;
+
+	if (on < 0)
+		on = env_int("ANNI_REVERSE", 1, 0, 1);
+	return on != 0;
+}
+
+/* ANNI_KEEP_MB: how much of the gradients' tail the sum of squares leaves in the memory-side cache. */
+static int keep_mb(void)
+{
+	static int mb = -1;
+
+	if (mb < 0)
+		mb = env_int("ANNI_KEEP_MB", 256, 0, 1 << 20);
+	return mb;
+}
+
 static bool aligned(const void *p, uintptr_t a)
 {
 	return ((uintptr_t)p & (a - 1)) == 0;
@@ -1203,6 +1267,21 @@ int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *parti
 	a.grad_scale = grad_scale;
 	a.partials = partials;
 	a.vec_ok = aligned(f.g, quad_bytes(f.grad_type)) ? 1 : 0;
+	{
+		/*
+		** The update that follows reads the gradients again.  What the sum reads last with
+		** ordinary loads stays in the memory-side cache (256 MiB on this part; streaming
+		** accesses pass it by), and the update, walking the flat from its end, finds it there.
+		*/
+		const int64_t n_tiles = (f.n + kTile - 1) / kTile;
+		const int64_t tile_bytes = kTile * (int64_t)(f.grad_type == kF32 ? 4 : f.grad_type == kBF16 ? 2 : 1);
+		const int64_t keep = (int64_t)keep_mb() * (1 << 20) / tile_bytes;
+		const int64_t round = (int64_t)grid * kSumsqFp8Ahead;
+
+		a.keep_from = n_tiles > keep ? n_tiles - keep : 0;
+		if (f.grad_type == kFP8)
+			a.keep_from = (a.keep_from + round - 1) / round * round;
+	}
 #define SUMSQ_LAUNCH(GT) \
 	do { \
 		if (nt_on()) \
@@ -1349,6 +1428,7 @@ int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double gra
 	a.clip = norm.clip;
 	a.state = norm.state;
 	a.der = f.der;
+	a.reverse = reverse_on() ? 1 : 0;
 	if (f.moment_type == kF32) {
 		if (f.grad_type == kF32)
 			update_launch<kF32, kF32>(st, grid, a);
