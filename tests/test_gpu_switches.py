@@ -1,0 +1,42 @@
+"""The tile walk and cache-hint switches of the step change where data is found, never a bit:
+sum of squares (two loops, changeover at any tile), update walking forward or backward, with
+non-temporal hints or without.  Each setting runs in a process of its own (the library reads its
+switches once), and all settings that share a grid must print the same digests."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+CHILD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "switch_child.py")
+
+
+def run_child(**switches):
+    env = {k: v for k, v in os.environ.items() if not k.startswith("ANNI_")}
+    env.update({k: str(v) for k, v in switches.items()})
+    r = subprocess.run([sys.executable, CHILD], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    line = [ln for ln in r.stdout.splitlines() if ln.startswith("DIGEST ")][-1]
+    return json.loads(line[7:])
+
+
+def test_default_grid(gpu):
+    want = run_child()
+    for gt in ("0", "1", "2"):
+        assert [row[1] for row in want[gt]].count(1) >= 1          # at least one clipped step
+        assert not any(row[6] for row in want[gt])                   # gradients cleared
+    assert run_child(ANNI_REVERSE=0, ANNI_KEEP_MB=0) == want
+    assert run_child(ANNI_NT=0, ANNI_PIPE=0) == want
+
+
+def test_one_workgroup_per_cu_changeover_inside_every_workgroup(gpu):
+    """256 workgroups over ~2200 tiles: each one takes 8 or 9 tiles, and with 5 MiB kept the
+    changeover from streaming to ordinary loads falls inside every workgroup's run (after one round
+    of the grid for fp8 codes)."""
+    want = run_child(ANNI_BLOCKS_PER_CU=1, ANNI_KEEP_MB=0)
+    assert run_child(ANNI_BLOCKS_PER_CU=1, ANNI_KEEP_MB=5) == want
+    assert run_child(ANNI_BLOCKS_PER_CU=1, ANNI_KEEP_MB=3, ANNI_REVERSE=0) == want
+    assert run_child(ANNI_BLOCKS_PER_CU=1, ANNI_KEEP_MB=100000) == want
