@@ -706,6 +706,13 @@ static void describe(const anni_adam *opt, Flat *f)
 	}
 }
 
+/* The ticket counter of the norm's second stage: in the 256 bytes reserved (and zeroed) for the state. */
+static unsigned int *ticket_word(const anni_adam_priv *pv)
+{
+	static_assert(sizeof(StepState) <= 128, "state and ticket share 256 bytes");
+	return (unsigned int *)((char *)pv->d_state + 128);
+}
+
 /* One step; ev (may be NULL) = four events recorded before, between and after the launches. */
 static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *ev)
 {
@@ -743,16 +750,18 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 	describe(opt, &f);
 	memset(&norm, 0, sizeof(norm));
 	norm.use_norm = (opt->grad_clip > 0.0 || opt->cfg.skip_nonfinite) ? 1 : 0;
-	norm.clip = opt->grad_clip > 0.0 ? opt->grad_clip : 0.0;
-	norm.skip_nonfinite = opt->cfg.skip_nonfinite;
 	norm.state = pv->d_state;
 	if (ev)
 		(void)hipEventRecord(ev[0], st);
 	if (norm.use_norm) {
-		if (launch_sumsq(st, f, grad_scale, pv->d_partials, &np) != 0)
+		SumsqFinish fin;
+
+		fin.ticket = ticket_word(pv);
+		fin.clip = opt->grad_clip > 0.0 ? opt->grad_clip : 0.0;
+		fin.skip_nonfinite = opt->cfg.skip_nonfinite;
+		fin.state = pv->d_state;
+		if (launch_sumsq(st, f, grad_scale, pv->d_partials, &np, &fin) != 0)
 			return -1;
-		norm.partials = pv->d_partials;
-		norm.n_partials = np;
 	}
 	if (ev)
 		(void)hipEventRecord(ev[1], st);

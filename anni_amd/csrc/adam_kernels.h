@@ -96,24 +96,30 @@ struct Flat {
 };
 
 /* How the update obtains the global norm (use_norm == 0: grad_scale is final). */
+/* The update takes its gradient scale and its skip decision from *state (use_norm) or from its arguments. */
 struct NormIn {
 	int		use_norm;
-	const double	*partials;
-	int		n_partials;
-	double		clip;
+	const StepState	*state;		/* stored by launch_sumsq with a SumsqFinish on the same stream */
+};
+
+/* Second stage of the norm inside the sum-of-squares launch. */
+struct SumsqFinish {
+	unsigned int	*ticket;	/* device word, zero between launches; one per partials array */
+	double		clip;		/* > 0: norm > clip scales the gradients by clip / (norm + 1e-12) */
 	int		skip_nonfinite;
-	StepState	*state;		/* may be NULL */
+	StepState	*state;		/* device or page-locked host memory */
 };
 
 /* Number of persistent workgroups for a flat of n elements on the current device. */
 int	grid_for(int64_t n);
 
-/* partials[0..*n_partials) = per-workgroup sums of (g * grad_scale)^2, fixed order. */
+/*
+** partials[0..*n_partials) = per-workgroup sums of (g * grad_scale)^2, fixed order.  With `fin`
+** the last workgroup to finish also folds them in index order into fin->state = {sum, sqrt,
+** clip-adjusted scale, flags}.
+*/
 int	launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *partials,
-		int *n_partials);
-/* state = {sum, sqrt, clip-adjusted scale, flags} from the partials, fixed order. */
-int	launch_finalize(hipStream_t st, const double *partials, int n_partials, double clip,
-		int skip_nonfinite, double grad_scale, StepState *state);
+		int *n_partials, const SumsqFinish *fin);
 int	launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double grad_scale,
 		const NormIn &norm);
 /*

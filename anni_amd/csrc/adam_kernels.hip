@@ -173,16 +173,6 @@ __device__ __forceinline__ double block_sum(double x, double *lds)
 	return total;
 }
 
-/* Second stage of the norm: the per-workgroup partials in index order, then block_sum. */
-__device__ __forceinline__ double partials_sum(const double *partials, int np, double *lds)
-{
-	double acc = 0.0;
-
-	for (int i = threadIdx.x; i < np; i += kThreads)
-		acc += partials[i];
-	return block_sum(acc, lds);
-}
-
 /* ---- derived outputs ------------------------------------------------------ */
 
 /* Max over the 64 lanes of a wavefront; lane 0 holds it. */
@@ -282,7 +272,78 @@ struct SumsqArgs {
 	double		*partials;
 	int		vec_ok;
 	int64_t		keep_from;	/* tiles from here on are read with ordinary (cacheable) loads */
+	/* second stage (ticket == NULL: partials only) */
+	unsigned int	*ticket;
+	double		clip;
+	int		skip_nonfinite;
+	StepState	*state;
 };
+
+/*
+** Second stage of the norm, inside the same launch: every workgroup stores its partial and
+** draws a ticket; the one that draws the last ticket knows that all partials are in memory, folds
+** them in index order -- the same sum whichever workgroup it is -- decides clip and skip, stores
+** the step state for the kernels that follow, and puts the ticket counter back to zero for the
+** next launch.  Nobody waits for anybody.  `state` may lie in page-locked host memory.
+**
+** The compute dies have a level-two cache each, so a release / acquire pair at device scope
+** writes back and invalidates whole caches -- 2048 of those at the end of the kernel were
+** measured at 0.1 ms.  Instead the partials themselves travel as device-scope atomic accesses,
+** which are performed where all dies see them: the partial is stored by an exchange whose result
+** the ticket increment consumes (so the increment cannot be issued before the exchange has been
+** performed), and the last workgroup reads the partials with atomic loads after its own increment
+** has returned.
+*/
+constexpr int kFoldAhead = 8;	/* partials a lane of the last workgroup has in flight */
+
+__device__ __forceinline__ void sumsq_finish(const SumsqArgs &a, double total, double *lds,
+	int *last)
+{
+	unsigned long long *cells = (unsigned long long *)a.partials;
+
+	if (threadIdx.x == 0) {
+		*last = 0;
+		if (a.ticket) {
+			const unsigned long long old = __hip_atomic_exchange(cells + blockIdx.x,
+			    (unsigned long long)__double_as_longlong(total), __ATOMIC_RELAXED,
+			    __HIP_MEMORY_SCOPE_AGENT);
+			unsigned int one = 1u;
+
+			/* ties the increment to the exchange's result: it waits for the exchange to return */
+			asm volatile("" : "+v"(one) : "v"(old));
+			*last = __hip_atomic_fetch_add(a.ticket, one, __ATOMIC_RELAXED,
+			    __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1u ? 1 : 0;
+		} else {
+			a.partials[blockIdx.x] = total;
+		}
+	}
+	__syncthreads();
+	if (!*last)
+		return;
+	/* lane l adds the partials l, l + 256, ... in that order, then the fixed tree over the lanes */
+	double acc = 0.0;
+
+	for (unsigned int i0 = threadIdx.x; i0 < gridDim.x; i0 += kFoldAhead * kThreads) {
+		unsigned long long raw[kFoldAhead];
+
+#pragma unroll
+		for (int k = 0; k < kFoldAhead; k++) {
+			const unsigned int i = i0 + (unsigned int)k * kThreads;
+
+			raw[k] = i < gridDim.x ? __hip_atomic_load(cells + i, __ATOMIC_RELAXED,
+			    __HIP_MEMORY_SCOPE_AGENT) : 0ull;
+		}
+#pragma unroll
+		for (int k = 0; k < kFoldAhead; k++)
+			if (i0 + (unsigned int)k * kThreads < gridDim.x)
+				acc += __longlong_as_double((long long)raw[k]);
+	}
+	const double ss = block_sum(acc, lds);
+
+	(void)norm_decide(ss, a.clip, a.skip_nonfinite, a.grad_scale, a.state, threadIdx.x == 0);
+	if (threadIdx.x == 0)
+		__hip_atomic_store(a.ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 /* The tiles first, first + step, ... below `stop`, added to the lane's four running sums. */
 template <int GT, bool NT>
@@ -349,6 +410,7 @@ template <int GT, bool NT>
 __global__ __launch_bounds__(kThreads) void sumsq_kernel(SumsqArgs a)
 {
 	__shared__ double lds[4];
+	__shared__ int last;
 	const int tid = threadIdx.x;
 	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
 	const int64_t keep_from = NT ? (a.keep_from < n_tiles ? a.keep_from : n_tiles) : 0;
@@ -359,8 +421,7 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(SumsqArgs a)
 	(void)sumsq_tiles<GT, false>(a, tile, gridDim.x, n_tiles, tid, acc);
 	const double total = block_sum((acc[0] + acc[1]) + (acc[2] + acc[3]), lds);
 
-	if (tid == 0)
-		a.partials[blockIdx.x] = total;
+	sumsq_finish(a, total, lds, &last);
 }
 
 /*
@@ -442,6 +503,7 @@ template <bool NT>
 __global__ __launch_bounds__(kThreads) void sumsq_fp8_kernel(SumsqArgs a)
 {
 	__shared__ double lds[4];
+	__shared__ int last;
 	const int tid = threadIdx.x;
 	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
 	const int64_t keep_from = NT ? (a.keep_from < n_tiles ? a.keep_from : n_tiles) : 0;
@@ -452,26 +514,7 @@ __global__ __launch_bounds__(kThreads) void sumsq_fp8_kernel(SumsqArgs a)
 	(void)sumsq_fp8_tiles<false>(a, t0, gridDim.x, n_tiles, n_tiles, tid, acc);
 	const double total = block_sum(acc, lds);
 
-	if (tid == 0)
-		a.partials[blockIdx.x] = total;
-}
-
-struct FinalizeArgs {
-	const double	*partials;
-	int		n_partials;
-	double		clip;
-	int		skip_nonfinite;
-	double		grad_scale;
-	StepState	*state;
-};
-
-__global__ __launch_bounds__(kThreads) void finalize_kernel(FinalizeArgs a)
-{
-	__shared__ double lds[4];
-	const double ss = partials_sum(a.partials, a.n_partials, lds);
-
-	(void)norm_decide(ss, a.clip, a.skip_nonfinite, a.grad_scale, a.state,
-	    threadIdx.x == 0);
+	sumsq_finish(a, total, lds, &last);
 }
 
 /* ---- the update ---------------------------------------------------------- */
@@ -491,13 +534,8 @@ struct UpdateArgs {
 	int		reverse;	/* walk the tiles from the last to the first */
 	StepConsts	c;
 	double		grad_scale;
-	/* norm */
-	int		use_norm;
-	int		skip_nonfinite;
-	const double	*partials;
-	int		n_partials;
-	double		clip;
-	StepState	*state;
+	int		use_norm;	/* scale and skip come from *state, stored by the sum of squares */
+	const StepState	*state;
 	Derived		der;
 };
 
@@ -542,23 +580,14 @@ __device__ __forceinline__ TileInfo tile_info(const UpdateArgs &a, int64_t turn,
 template <int GT, int MT, int U, bool NT, bool DER>
 __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 {
-	__shared__ double lds[4];
 	const int tid = threadIdx.x;
 	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
 	double gs = a.grad_scale;
 	bool skip = false;
 
 	if (a.use_norm) {
-		/*
-		** Every workgroup folds the same partials in the same order, so all of
-		** them derive the same scale without any cross-workgroup handshake.
-		*/
-		const double ss = partials_sum(a.partials, a.n_partials, lds);
-		const NormOut o = norm_decide(ss, a.clip, a.skip_nonfinite, gs, a.state,
-		    blockIdx.x == 0 && tid == 0);
-
-		gs = o.gs;
-		skip = o.skip;
+		gs = a.state->grad_scale;
+		skip = a.state->skipped != 0;
 	}
 	TileInfo cur = tile_info<GT>(a, blockIdx.x < n_tiles ? (int64_t)blockIdx.x : 0, skip);
 
@@ -820,7 +849,6 @@ __device__ __forceinline__ void half_consume(const HalfStage<GT, MT> &st, const 
 template <int GT, int MT, bool NT, bool DER>
 __global__ __launch_bounds__(kThreads) void adam_update_pipe_kernel(UpdateArgs a)
 {
-	__shared__ double lds[4];
 	const int tid = threadIdx.x;
 	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
 	const int64_t step = gridDim.x;
@@ -831,12 +859,8 @@ __global__ __launch_bounds__(kThreads) void adam_update_pipe_kernel(UpdateArgs a
 	int64_t tile = blockIdx.x;
 
 	if (a.use_norm) {
-		const double ss = partials_sum(a.partials, a.n_partials, lds);
-		const NormOut o = norm_decide(ss, a.clip, a.skip_nonfinite, gs, a.state,
-		    blockIdx.x == 0 && tid == 0);
-
-		gs = o.gs;
-		skip = o.skip;
+		gs = a.state->grad_scale;
+		skip = a.state->skipped != 0;
 	}
 	if (tile >= n_tiles)
 		return;
@@ -1251,7 +1275,7 @@ static int check_flat(const Flat &f, bool need_state)
 }
 
 int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *partials,
-	int *n_partials)
+	int *n_partials, const SumsqFinish *fin)
 {
 	SumsqArgs a;
 	int grid;
@@ -1266,6 +1290,18 @@ int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *parti
 	a.gscale = f.gscale;
 	a.grad_scale = grad_scale;
 	a.partials = partials;
+	a.ticket = nullptr;
+	a.clip = 0.0;
+	a.skip_nonfinite = 0;
+	a.state = nullptr;
+	if (fin) {
+		if (!fin->ticket || !fin->state)
+			return -1;
+		a.ticket = fin->ticket;
+		a.clip = fin->clip;
+		a.skip_nonfinite = fin->skip_nonfinite;
+		a.state = fin->state;
+	}
 	a.vec_ok = aligned(f.g, quad_bytes(f.grad_type)) ? 1 : 0;
 	{
 		/*
@@ -1302,23 +1338,6 @@ int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *parti
 	}
 #undef SUMSQ_LAUNCH
 	*n_partials = grid;
-	return hipGetLastError() == hipSuccess ? 0 : -1;
-}
-
-int launch_finalize(hipStream_t st, const double *partials, int n_partials, double clip,
-	int skip_nonfinite, double grad_scale, StepState *state)
-{
-	FinalizeArgs a;
-
-	if (!partials || n_partials <= 0 || !state)
-		return -1;
-	a.partials = partials;
-	a.n_partials = n_partials;
-	a.clip = clip;
-	a.skip_nonfinite = skip_nonfinite;
-	a.grad_scale = grad_scale;
-	a.state = state;
-	hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kThreads), 0, st, a);
 	return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -1379,6 +1398,30 @@ static void update_launch(hipStream_t st, int grid, const UpdateArgs &a)
 	}
 }
 
+/*
+** Workgroups of the update.  Compute units do not stream at one speed (where their data lie,
+** what shares their part of the chip), so a grid in which every workgroup owns an equal share of
+** the flat ends as fast as its slowest member.  With many more workgroups than fit the chip at
+** once the dispatcher hands the next one to whichever compute unit falls free: measured best at
+** two tiles per workgroup (-2.8 % against eight resident workgroups per compute unit; -6.5 % on a
+** placement that was slow to begin with), eight with bf16 moments, whose kernel lives on having a
+** next tile to prefetch.  ANNI_TILES_PER_WG sets the number; 0 = the resident grid.
+*/
+static int update_grid(int64_t n, bool bf16_moments)
+{
+	static int per = -2;
+	const int64_t tiles = (n + kTile - 1) / kTile;
+	int grid = grid_for(n);
+	int k;
+
+	if (per == -2)
+		per = env_int("ANNI_TILES_PER_WG", -1, -1, 1 << 20);
+	k = per >= 0 ? per : (bf16_moments ? 8 : 2);
+	if (k > 0 && tiles / k > grid)
+		grid = (int)(tiles / k);
+	return grid;
+}
+
 /* Derived outputs need the launch table, an 8-byte aligned pack flat and descriptors for it. */
 static int check_derived(const Flat &f)
 {
@@ -1401,9 +1444,9 @@ int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double gra
 
 	if (check_flat(f, true) != 0 || check_derived(f) != 0)
 		return -1;
-	if (norm.use_norm && (!norm.partials || norm.n_partials <= 0))
+	if (norm.use_norm && !norm.state)
 		return -1;
-	grid = grid_for(f.n);
+	grid = update_grid(f.n, f.moment_type == kBF16);
 	a.p = f.p;
 	a.g = f.g;
 	a.m = f.m;
@@ -1422,10 +1465,6 @@ int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double gra
 	a.c = c;
 	a.grad_scale = grad_scale;
 	a.use_norm = norm.use_norm;
-	a.skip_nonfinite = norm.skip_nonfinite;
-	a.partials = norm.partials;
-	a.n_partials = norm.n_partials;
-	a.clip = norm.clip;
 	a.state = norm.state;
 	a.der = f.der;
 	a.reverse = reverse_on() ? 1 : 0;

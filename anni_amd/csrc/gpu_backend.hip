@@ -281,7 +281,9 @@ static bool scratch_ready(void)
 	void *d = nullptr;
 	void *h = nullptr;
 
-	if (hipMalloc(&d, sizeof(double) * kMaxPartials) != hipSuccess
+	/* the partials and, behind them, the ticket counter of the second stage */
+	if (hipMalloc(&d, sizeof(double) * kMaxPartials + 256) != hipSuccess
+	    || hipMemset(d, 0, sizeof(double) * kMaxPartials + 256) != hipSuccess
 	    || hipHostMalloc(&h, sizeof(StepState), hipHostMallocDefault) != hipSuccess) {
 		(void)hipGetLastError();
 		if (d)
@@ -776,9 +778,14 @@ int gpu_grad_sumsq(const ann_real *d_x, int n, double *out)
 	{
 		ProfScope prof(0);
 
-		/* the one-workgroup second stage stores its result straight into page-locked host memory */
-		if (launch_sumsq(g_stream, f, 1.0, g_partials, &np) != 0
-		    || launch_finalize(g_stream, g_partials, np, 0.0, 0, 1.0, g_host_state) != 0)
+		SumsqFinish fin;
+
+		/* the second stage stores its result straight into page-locked host memory */
+		fin.ticket = (unsigned int *)(g_partials + kMaxPartials);
+		fin.clip = 0.0;
+		fin.skip_nonfinite = 0;
+		fin.state = g_host_state;
+		if (launch_sumsq(g_stream, f, 1.0, g_partials, &np, &fin) != 0)
 			return -1;
 	}
 	if (!hip_ok(sync_stream_and_deliver(), "sumsq sync"))
