@@ -339,6 +339,55 @@ def test_device_normal_generator_and_bf16_convert(gpu, oracle):
     assert (h.download(np.uint16, n) == oracle.bf16_rne(x)).all()
 
 
+def test_steps_back_to_back_equal_steps_with_a_sync_between(gpu):
+    """Eight steps queued in one go (sum of squares, second stage in its last workgroup, update,
+    again and again with nothing in between) against the same eight steps with a host
+    synchronisation after each: a second stage that read a partial too early, or one left from the
+    step before, would change the clip scale and with it every element."""
+    import ctypes as C
+    tensors = [(4096 * 1500 + 7, 3), (1536, 0), (4096 * 700, 3), (3, 1)]
+    rng = np.random.default_rng(31)
+    steps = 8
+    runs = []
+    p0 = grads = None
+    for mode in ("queued", "synced"):
+        opt = make(gpu, tensors, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True,
+                   grad_slots=steps)
+        n = opt.n
+        if p0 is None:
+            p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
+            # norms 0.3 .. 2.4 around the clip at 1.0
+            grads = [(rng.standard_normal(n) * ((0.3 + 0.3 * k) / np.sqrt(n))).astype(np.float32)
+                     for k in range(steps)]
+        opt.upload("param", p0)
+        opt.seed_twins()
+        slots = [opt.grad_slot(k) for k in range(steps)]
+        for k in range(steps):
+            assert gpu.gpu_memcpy_h2d(slots[k], grads[k].ctypes.data, grads[k].nbytes) == 0
+        assert gpu.gpu_stream_sync() == 0
+        lrs = [1e-3 * (k + 1) for k in range(steps)]
+        if mode == "queued":
+            ms = C.c_float(0)
+            assert gpu.anni_adam_time_steps(opt.h, steps, (C.c_void_p * steps)(*slots), steps,
+                                            (C.c_double * steps)(*lrs),
+                                            (C.c_double * steps)(*[1.0] * steps), C.byref(ms),
+                                            None, None) == 0
+        else:
+            for k in range(steps):
+                opt.bind_grad(slots[k])
+                opt.step_scaled(lrs[k])
+                st = opt.sync_stats()
+                assert st.last_clipped == (1 if 0.3 + 0.3 * k > 1.0 else 0), k
+        st = opt.sync_stats()
+        runs.append((opt.download("param"), opt.download("m"), opt.download("v"),
+                     opt.download("twin"), st.last_sumsq, opt.t))
+        opt.free()
+    a, b = runs
+    assert a[4] == b[4] and a[5] == b[5] == steps
+    for x, y in zip(a[:4], b[:4]):
+        assert same_bits(x, y)
+
+
 def test_two_optimizers_side_by_side(gpu, oracle):
     """Two arenas with different storage modes stepping in turn share the stream and the
     library's state and do not disturb each other."""

@@ -102,6 +102,30 @@ def test_grad_sumsq_unaligned_and_nonfinite(gpu, oracle):
         assert not math.isfinite(out.value)
 
 
+def test_grad_sumsq_back_to_back_on_changing_inputs(gpu, oracle):
+    """The second stage of the sum runs inside the same launch: the last workgroup to finish
+    folds the partials of all the others.  Launches back to back on inputs of different content and
+    size must each return their own sum, to the bit, every time -- a partial left over from the
+    launch before, or one not yet visible, would show."""
+    rng = np.random.default_rng(2048)
+    cases = []
+    for n, scale in ((4096 * 2075 + 17, 3e-2), (3000017, 1.0), (4096 * 2048, 1e-3), (5, 2.0)):
+        g = (rng.standard_normal(n) * scale).astype(np.float32)
+        want = oracle.sumsq(g)
+        cases.append((dev(gpu, g), n, want))
+    out = C.c_double(0)
+    first = []
+    for d, n, want in cases:
+        assert gpu.gpu_grad_sumsq(d.ptr, n, C.byref(out)) == 0
+        assert abs(out.value - want) <= 1e-11 * want
+        first.append(out.value)
+    order = rng.integers(0, len(cases), 1500)
+    for k in order:
+        d, n, _want = cases[k]
+        assert gpu.gpu_grad_sumsq(d.ptr, n, C.byref(out)) == 0
+        assert out.value == first[k], (k, out.value, first[k])
+
+
 class FlatState:
     """p/g/m/v/twin on the device + the same on the host for the oracle."""
 
