@@ -1405,9 +1405,10 @@ static void update_launch(hipStream_t st, int grid, const UpdateArgs &a)
 ** once the dispatcher hands the next one to whichever compute unit falls free: measured best at
 ** two tiles per workgroup (-2.8 % against eight resident workgroups per compute unit; -6.5 % on a
 ** placement that was slow to begin with), eight with bf16 moments, whose kernel lives on having a
-** next tile to prefetch.  ANNI_TILES_PER_WG sets the number; 0 = the resident grid.
+** next tile to prefetch, one for the kernels with derived outputs and for the E4M3 pass (-9 %).
+** ANNI_TILES_PER_WG sets the number for all of them; 0 = the resident grid.
 */
-static int update_grid(int64_t n, bool bf16_moments)
+static int balanced_grid(int64_t n, int tiles_per_wg)
 {
 	static int per = -2;
 	const int64_t tiles = (n + kTile - 1) / kTile;
@@ -1416,10 +1417,15 @@ static int update_grid(int64_t n, bool bf16_moments)
 
 	if (per == -2)
 		per = env_int("ANNI_TILES_PER_WG", -1, -1, 1 << 20);
-	k = per >= 0 ? per : (bf16_moments ? 8 : 2);
+	k = per >= 0 ? per : tiles_per_wg;
 	if (k > 0 && tiles / k > grid)
 		grid = (int)(tiles / k);
 	return grid;
+}
+
+static int update_grid(int64_t n, bool bf16_moments, bool derived)
+{
+	return balanced_grid(n, bf16_moments ? 8 : derived ? 1 : 2);
 }
 
 /* Derived outputs need the launch table, an 8-byte aligned pack flat and descriptors for it. */
@@ -1446,7 +1452,7 @@ int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double gra
 		return -1;
 	if (norm.use_norm && !norm.state)
 		return -1;
-	grid = update_grid(f.n, f.moment_type == kBF16);
+	grid = update_grid(f.n, f.moment_type == kBF16, f.der.wamax != nullptr || f.der.pack != nullptr);
 	a.p = f.p;
 	a.g = f.g;
 	a.m = f.m;
@@ -1566,9 +1572,9 @@ int launch_fp8_twins(hipStream_t st, const Flat &f, uint8_t *q, float *wscale,
 	a.state = state;
 	a.vec_ok = aligned(f.p, 16) && aligned(q, 4) ? 1 : 0;
 	if (nt_on())
-		hipLaunchKernelGGL((fp8_twin_kernel<true>), dim3(grid_for(f.n)), dim3(kThreads), 0, st, a);
+		hipLaunchKernelGGL((fp8_twin_kernel<true>), dim3(balanced_grid(f.n, 1)), dim3(kThreads), 0, st, a);
 	else
-		hipLaunchKernelGGL((fp8_twin_kernel<false>), dim3(grid_for(f.n)), dim3(kThreads), 0, st, a);
+		hipLaunchKernelGGL((fp8_twin_kernel<false>), dim3(balanced_grid(f.n, 1)), dim3(kThreads), 0, st, a);
 	return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
