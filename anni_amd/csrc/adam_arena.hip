@@ -20,6 +20,9 @@
 
 using namespace anni;
 
+/* Step state (128 bytes) + the ticket counters of the norm's second stage. */
+static const size_t kStateBytes = 128 + ((kTicketBytes + 255) / 256) * 256;
+
 struct anni_adam_priv {
 	void			*arena;
 	size_t			arena_bytes;
@@ -138,7 +141,7 @@ static bool place(const Sizes &z, bool spread, Placement *pl)
 	const size_t tables = round_up((size_t)z.n_tensors * sizeof(float), 256)
 	    + round_up((size_t)z.n_tensors * sizeof(Seg), 256)
 	    + round_up((size_t)z.n_tiles * sizeof(int32_t), 256)
-	    + round_up((size_t)kMaxPartials * sizeof(double), 256) + 256;
+	    + round_up((size_t)kMaxPartials * sizeof(double), 256) + kStateBytes;
 
 	memset(pl, 0, sizeof(*pl));
 	if (spread) {
@@ -166,7 +169,7 @@ static bool place(const Sizes &z, bool spread, Placement *pl)
 	pl->off_state = pl->off_part + round_up((size_t)kMaxPartials * sizeof(double), 256);
 	pl->spread = spread ? 1 : 0;
 	if (spread) {
-		pl->hole_off = round_up(pl->off_state + 256, big);
+		pl->hole_off = round_up(pl->off_state + kStateBytes, big);
 		pl->hole_bytes = 4 * stride > pl->hole_off ? 4 * stride - pl->hole_off : 0;
 	}
 	if (hipMalloc(&pl->arena, pl->total) != hipSuccess) {
@@ -218,7 +221,7 @@ static bool init_contents(anni_adam *opt, const Sizes &z, const Placement &pl,
 	    && (!z.tw_bytes || launch_fill_bytes(st, base + pl.off_twin, 0, z.tw_bytes) == 0)
 	    && (!z.n_slots || launch_fill_bytes(st, base + pl.off_g, 0,
 	    (size_t)z.n_slots * z.g_bytes) == 0)
-	    && launch_fill_bytes(st, base + pl.off_part, 0, pl.off_state + 256 - pl.off_part) == 0
+	    && launch_fill_bytes(st, base + pl.off_part, 0, pl.off_state + kStateBytes - pl.off_part) == 0
 	    && hip_ok(hipMemcpyAsync(opt->d_gscale, ones.data(), (size_t)z.n_tensors * sizeof(float),
 	    hipMemcpyHostToDevice, st), "gscale")
 	    && hip_ok(hipMemcpyAsync(opt->priv->d_segs, segs.data(), (size_t)z.n_tensors * sizeof(Seg),
@@ -706,10 +709,10 @@ static void describe(const anni_adam *opt, Flat *f)
 	}
 }
 
-/* The ticket counter of the norm's second stage: in the 256 bytes reserved (and zeroed) for the state. */
+/* The ticket counters of the norm's second stage lie behind the step state (reserved and zeroed with it). */
 static unsigned int *ticket_word(const anni_adam_priv *pv)
 {
-	static_assert(sizeof(StepState) <= 128, "state and ticket share 256 bytes");
+	static_assert(sizeof(StepState) <= 128, "the tickets start 128 bytes behind the state");
 	return (unsigned int *)((char *)pv->d_state + 128);
 }
 

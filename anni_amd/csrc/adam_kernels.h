@@ -102,9 +102,18 @@ struct NormIn {
 	const StepState	*state;		/* stored by launch_sumsq with a SumsqFinish on the same stream */
 };
 
+/*
+** Ticket counters of the norm's second stage: one per group of workgroups and one above them,
+** each on a 128-byte line of its own.  kTicketBytes of device memory, zero between launches, one
+** block per partials array.
+*/
+constexpr int kTicketGroups = 64;
+constexpr int kTicketStride = 32;		/* in words */
+constexpr size_t kTicketBytes = (size_t)(1 + kTicketGroups) * kTicketStride * sizeof(unsigned int);
+
 /* Second stage of the norm inside the sum-of-squares launch. */
 struct SumsqFinish {
-	unsigned int	*ticket;	/* device word, zero between launches; one per partials array */
+	unsigned int	*ticket;	/* kTicketBytes, 128-byte aligned */
 	double		clip;		/* > 0: norm > clip scales the gradients by clip / (norm + 1e-12) */
 	int		skip_nonfinite;
 	StepState	*state;		/* device or page-locked host memory */

@@ -281,9 +281,9 @@ static bool scratch_ready(void)
 	void *d = nullptr;
 	void *h = nullptr;
 
-	/* the partials and, behind them, the ticket counter of the second stage */
-	if (hipMalloc(&d, sizeof(double) * kMaxPartials + 256) != hipSuccess
-	    || hipMemset(d, 0, sizeof(double) * kMaxPartials + 256) != hipSuccess
+	/* the partials and, behind them, the ticket counters of the second stage */
+	if (hipMalloc(&d, sizeof(double) * kMaxPartials + kTicketBytes) != hipSuccess
+	    || hipMemset(d, 0, sizeof(double) * kMaxPartials + kTicketBytes) != hipSuccess
 	    || hipHostMalloc(&h, sizeof(StepState), hipHostMallocDefault) != hipSuccess) {
 		(void)hipGetLastError();
 		if (d)
