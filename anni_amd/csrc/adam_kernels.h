@@ -119,7 +119,7 @@ struct SumsqFinish {
 	StepState	*state;		/* device or page-locked host memory */
 };
 
-/* Number of persistent workgroups for a flat of n elements on the current device. */
+/* Workgroups of a resident grid for a flat of n elements on the current device. */
 int	grid_for(int64_t n);
 
 /*

@@ -2,8 +2,8 @@
 ** gfx950 kernels of the AnnI optimizer step: the global sum of squares (clip
 ** norm), the fused AdamW update with bf16 twin emission, and the small helpers
 ** around them.  Everything here is a memory-bound stream: 64-lane wavefronts,
-** 16-byte accesses per lane where the element type allows, persistent
-** workgroups striding over tiles, no matrix cores.
+** 16-byte accesses per lane where the element type allows, workgroups
+** striding over tiles of 4096 elements, no matrix cores.
 **
 ** Replaces (does not port) the reference's device step, num/gpu_cuda.cu:8417-8712:
 ** the arithmetic follows the reference's HOST loop (lang/lm_adam.c:571-598) in
@@ -1210,7 +1210,7 @@ static int cu_count(void)
 	return cus;
 }
 
-/* ANNI_BLOCKS_PER_CU: persistent workgroups per compute unit (default 8). */
+/* ANNI_BLOCKS_PER_CU: workgroups per compute unit of a grid that is resident as a whole (default 8). */
 int grid_for(int64_t n)
 {
 	static int per_cu;
