@@ -587,9 +587,10 @@ __device__ __forceinline__ TileInfo tile_info(const UpdateArgs &a, int64_t turn,
 }
 
 /*
-** U = quads a lane keeps in flight at once (kQuadsPerTile % U == 0).  With narrow storage
-** types the kernel moves fewer bytes per element for the same arithmetic, so those modes
-** take the cheaper constant division (adam_math.h) and the deeper unroll.
+** U = quads a lane keeps in flight at once (kQuadsPerTile % U == 0); the whole tile in every mode
+** (half the tile was measured 0.5 % slower in the all-f32 mode).  With narrow storage types the
+** kernel moves fewer bytes per element for the same arithmetic, so those modes take the cheaper
+** constant division (adam_math.h).
 */
 template <int GT, int MT, int U, bool NT, bool DER>
 __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
@@ -1356,7 +1357,7 @@ int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *parti
 }
 
 #ifndef ANNI_UPDATE_UNROLL
-#define ANNI_UPDATE_UNROLL 2		/* all-f32 mode */
+#define ANNI_UPDATE_UNROLL 4		/* all-f32 mode: the whole tile in flight */
 #endif
 #ifndef ANNI_UPDATE_UNROLL_NARROW
 #define ANNI_UPDATE_UNROLL_NARROW 4	/* bf16 moments / bf16 or fp8 gradients */
@@ -1416,11 +1417,12 @@ static void update_launch(hipStream_t st, int grid, const UpdateArgs &a)
 ** Workgroups of the update.  Compute units do not stream at one speed (where their data lie,
 ** what shares their part of the chip), so a grid in which every workgroup owns an equal share of
 ** the flat ends as fast as its slowest member.  With many more workgroups than fit the chip at
-** once the dispatcher hands the next one to whichever compute unit falls free: measured best at
-** two tiles per workgroup (-2.8 % against eight resident workgroups per compute unit; -6.5 % on a
-** placement that was slow to begin with), eight with bf16 moments, whose kernel lives on having a
-** next tile to prefetch, one for the kernels with derived outputs and for the E4M3 pass (-9 %).
-** ANNI_TILES_PER_WG sets the number for all of them; 0 = the resident grid.
+** once the dispatcher hands the next one to whichever compute unit falls free: -3 to -4 % against
+** eight resident workgroups per compute unit (-6.5 % on a placement that was slow to begin with).
+** Measured best: one tile per workgroup in the all-f32 mode, whose lanes have the whole tile in
+** flight, for the kernels with derived outputs and for the E4M3 pass; two for the pipelined kernel
+** with narrow gradients; eight with bf16 moments, whose kernel lives on having a next tile to
+** prefetch.  ANNI_TILES_PER_WG sets the number for all of them; 0 = the resident grid.
 */
 static int balanced_grid(int64_t n, int tiles_per_wg)
 {
@@ -1437,9 +1439,12 @@ static int balanced_grid(int64_t n, int tiles_per_wg)
 	return grid;
 }
 
-static int update_grid(int64_t n, bool bf16_moments, bool derived)
+static int update_grid(const Flat &f)
 {
-	return balanced_grid(n, bf16_moments ? 8 : derived ? 1 : 2);
+	const bool derived = f.der.wamax != nullptr || f.der.pack != nullptr;
+	const bool all_f32 = f.grad_type == kF32 && f.moment_type == kF32;
+
+	return balanced_grid(f.n, f.moment_type == kBF16 ? 8 : (derived || all_f32) ? 1 : 2);
 }
 
 /* Derived outputs need the launch table, an 8-byte aligned pack flat and descriptors for it. */
@@ -1466,7 +1471,7 @@ int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double gra
 		return -1;
 	if (norm.use_norm && !norm.state)
 		return -1;
-	grid = update_grid(f.n, f.moment_type == kBF16, f.der.wamax != nullptr || f.der.pack != nullptr);
+	grid = update_grid(f);
 	a.p = f.p;
 	a.g = f.g;
 	a.m = f.m;
