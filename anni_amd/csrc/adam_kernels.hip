@@ -1417,12 +1417,10 @@ static void update_launch(hipStream_t st, int grid, const UpdateArgs &a)
 ** Workgroups of the update.  Compute units do not stream at one speed (where their data lie,
 ** what shares their part of the chip), so a grid in which every workgroup owns an equal share of
 ** the flat ends as fast as its slowest member.  With many more workgroups than fit the chip at
-** once the dispatcher hands the next one to whichever compute unit falls free: -3 to -4 % against
-** eight resident workgroups per compute unit (-6.5 % on a placement that was slow to begin with).
-** Measured best: one tile per workgroup in the all-f32 mode, whose lanes have the whole tile in
-** flight, for the kernels with derived outputs and for the E4M3 pass; two for the pipelined kernel
-** with narrow gradients; eight with bf16 moments, whose kernel lives on having a next tile to
-** prefetch.  ANNI_TILES_PER_WG sets the number for all of them; 0 = the resident grid.
+** once the dispatcher hands the next one to whichever compute unit falls free: -4 to -6 % against
+** eight resident workgroups per compute unit.  Measured best in every storage mode, for the kernels
+** with derived outputs and for the E4M3 pass: one tile per workgroup.  ANNI_TILES_PER_WG sets
+** another number for all of them; 0 = the resident grid.
 */
 static int balanced_grid(int64_t n, int tiles_per_wg)
 {
@@ -1437,14 +1435,6 @@ static int balanced_grid(int64_t n, int tiles_per_wg)
 	if (k > 0 && tiles / k > grid)
 		grid = (int)(tiles / k);
 	return grid;
-}
-
-static int update_grid(const Flat &f)
-{
-	const bool derived = f.der.wamax != nullptr || f.der.pack != nullptr;
-	const bool all_f32 = f.grad_type == kF32 && f.moment_type == kF32;
-
-	return balanced_grid(f.n, f.moment_type == kBF16 ? 8 : (derived || all_f32) ? 1 : 2);
 }
 
 /* Derived outputs need the launch table, an 8-byte aligned pack flat and descriptors for it. */
@@ -1471,7 +1461,7 @@ int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double gra
 		return -1;
 	if (norm.use_norm && !norm.state)
 		return -1;
-	grid = update_grid(f);
+	grid = balanced_grid(f.n, 1);
 	a.p = f.p;
 	a.g = f.g;
 	a.m = f.m;
