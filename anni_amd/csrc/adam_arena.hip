@@ -716,7 +716,10 @@ static unsigned int *ticket_word(const anni_adam_priv *pv)
 	return (unsigned int *)((char *)pv->d_state + 128);
 }
 
-/* One step; ev (may be NULL) = four events recorded before, between and after the launches. */
+/*
+** One step; ev (may be NULL) = four events recorded before the step, after the sum of squares, after
+** the update and after the derived outputs; an entry that is NULL is not recorded.
+*/
 static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *ev)
 {
 	anni_adam_priv *pv;
@@ -754,7 +757,7 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 	memset(&norm, 0, sizeof(norm));
 	norm.use_norm = (opt->grad_clip > 0.0 || opt->cfg.skip_nonfinite) ? 1 : 0;
 	norm.state = pv->d_state;
-	if (ev)
+	if (ev && ev[0])
 		(void)hipEventRecord(ev[0], st);
 	if (norm.use_norm) {
 		SumsqFinish fin;
@@ -766,7 +769,7 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 		if (launch_sumsq(st, f, grad_scale, pv->d_partials, &np, &fin) != 0)
 			return -1;
 	}
-	if (ev)
+	if (ev && ev[1])
 		(void)hipEventRecord(ev[1], st);
 	/*
 	** The words the update raises start every step at zero, cleared on the stream by a fill
@@ -779,7 +782,7 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 	if (launch_update(st, f, c, grad_scale, norm) != 0)
 		return -1;
 	opt->t = t;
-	if (ev)
+	if (ev && ev[2])
 		(void)hipEventRecord(ev[2], st);
 	if (pv->fp8_twins) {
 		if (launch_amax_fold(st, f, norm.use_norm ? pv->d_state : nullptr) != 0)
@@ -788,7 +791,7 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 		    opt->n_tensors, norm.use_norm ? pv->d_state : nullptr) != 0)
 			return -1;
 	}
-	if (ev)
+	if (ev && ev[3])
 		(void)hipEventRecord(ev[3], st);
 	/*
 	** The weights moved: consumers that cache derived copies keyed on the weight epoch rebuild
@@ -845,7 +848,16 @@ static int time_steps_body(anni_adam *opt, int count, void *const *grads, int n_
 	if (grads && n_grads <= 0)
 		return -1;
 	st = compute_stream();
-	ev.resize(per_kernel ? (size_t)count * 4 : 2);
+	/*
+	** Per kernel: ev[0] before the first step, then per step the events after the sum of squares,
+	** after the update and (only with derived outputs) after those; a step begins where the one
+	** before ended.  Every record costs the stream a few microseconds between two kernels, so
+	** there is none that is not read.
+	*/
+	const bool derived = opt->priv && opt->priv->fp8_twins;
+	const size_t per_step = derived ? 3 : 2;
+
+	ev.resize(per_kernel ? (size_t)count * per_step + 1 : 2);
 	for (size_t i = 0; i < ev.size(); i++)
 		if (hipEventCreate(&ev[i]) != hipSuccess) {
 			for (size_t k = 0; k < i; k++)
@@ -855,9 +867,19 @@ static int time_steps_body(anni_adam *opt, int count, void *const *grads, int n_
 	if (!per_kernel)
 		(void)hipEventRecord(ev[0], st);
 	for (int i = 0; i < count && rc == 0; i++) {
+		hipEvent_t four[4] = { nullptr, nullptr, nullptr, nullptr };
+
+		if (per_kernel) {
+			const size_t at = 1 + (size_t)i * per_step;
+
+			four[0] = i == 0 ? ev[0] : nullptr;
+			four[1] = ev[at];
+			four[2] = ev[at + 1];
+			four[3] = derived ? ev[at + 2] : nullptr;
+		}
 		if (grads)
 			(void)anni_adam_bind_grad(opt, grads[i % n_grads]);
-		rc = step_impl(opt, lr[i], grad_scale[i], per_kernel ? &ev[(size_t)i * 4] : nullptr);
+		rc = step_impl(opt, lr[i], grad_scale[i], per_kernel ? four : nullptr);
 		if (rc == 1)
 			rc = -1;		/* a timed run must not contain no-op steps */
 	}
@@ -872,17 +894,19 @@ static int time_steps_body(anni_adam *opt, int count, void *const *grads, int n_
 			float a = 0.0f, b = 0.0f, d = 0.0f;
 
 			for (int i = 0; i < count; i++) {
+				const size_t at = 1 + (size_t)i * per_step;
 				float x = 0.0f, y = 0.0f, w = 0.0f;
 
-				(void)hipEventElapsedTime(&x, ev[(size_t)i * 4], ev[(size_t)i * 4 + 1]);
-				(void)hipEventElapsedTime(&y, ev[(size_t)i * 4 + 1], ev[(size_t)i * 4 + 2]);
-				(void)hipEventElapsedTime(&w, ev[(size_t)i * 4 + 2], ev[(size_t)i * 4 + 3]);
+				(void)hipEventElapsedTime(&x, ev[at - 1], ev[at]);
+				(void)hipEventElapsedTime(&y, ev[at], ev[at + 1]);
+				if (derived)
+					(void)hipEventElapsedTime(&w, ev[at + 1], ev[at + 2]);
 				a += x;
 				b += y;
 				d += w;
 			}
 			opt->priv->der_ms = d;
-			(void)hipEventElapsedTime(&ms, ev[0], ev[(size_t)count * 4 - 1]);
+			(void)hipEventElapsedTime(&ms, ev[0], ev[ev.size() - 1]);
 			if (ms_sumsq)
 				*ms_sumsq = a;
 			if (ms_update)
