@@ -30,6 +30,8 @@ def test_default_grid(gpu):
         assert not any(row[6] for row in want[gt])                   # gradients cleared
     assert run_child(ANNI_REVERSE=0, ANNI_KEEP_MB=0) == want
     assert run_child(ANNI_NT=0, ANNI_PIPE=0) == want
+    assert run_child(ANNI_TILES_PER_WG=0) == want            # the resident grid
+    assert run_child(ANNI_TILES_PER_WG=3, ANNI_PIPE=2) == want
 
 
 def test_one_workgroup_per_cu_changeover_inside_every_workgroup(gpu):
