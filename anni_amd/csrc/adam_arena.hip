@@ -1228,6 +1228,11 @@ void anni_gpu_set_stream(void *hip_stream)
 		set_compute_stream((hipStream_t)hip_stream);
 }
 
+void anni_gpu_reload_switches(void)
+{
+	reload_switches();
+}
+
 int anni_gpu_device_info(char *name, size_t cap, int *driver_version)
 {
 	hipDeviceProp_t prop;

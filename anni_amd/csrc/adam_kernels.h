@@ -119,6 +119,9 @@ struct SumsqFinish {
 	StepState	*state;		/* device or page-locked host memory */
 };
 
+/* Reads the ANNI_* tuning switches from the environment again (they are read once, on first use). */
+void	reload_switches(void);
+
 /* Workgroups of a resident grid for a flat of n elements on the current device. */
 int	grid_for(int64_t n);
 

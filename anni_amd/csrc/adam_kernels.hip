@@ -1171,6 +1171,40 @@ static int env_int(const char *name, int dflt, int lo, int hi)
 	return v;
 }
 
+/*
+** The tuning switches, read from the environment on first use and again whenever
+** reload_switches() is called (a sweep that compares settings on one arena in one process: two
+** processes differ by what memory they were given, by more than most settings do).
+*/
+struct Switches {
+	int	loaded;
+	int	blocks_per_cu;	/* ANNI_BLOCKS_PER_CU: workgroups per compute unit of a grid that is resident as a whole */
+	int	nt;		/* ANNI_NT=0: no streaming (non-temporal) cache hints */
+	int	reverse;	/* ANNI_REVERSE=0: the update walks the tiles from the first to the last */
+	int	keep_mb;	/* ANNI_KEEP_MB: how much of the gradients' tail the sum of squares leaves in the memory-side cache */
+	int	pipe;		/* ANNI_PIPE=0: narrow storage modes on the plain kernel; 2: the all-f32 mode pipelined too */
+	int	tiles_per_wg;	/* ANNI_TILES_PER_WG: tiles per workgroup of the update; 0 = the resident grid; -1 = the default */
+};
+static Switches g_sw;
+
+void reload_switches(void)
+{
+	g_sw.blocks_per_cu = env_int("ANNI_BLOCKS_PER_CU", 8, 1, 32);
+	g_sw.nt = env_int("ANNI_NT", 1, 0, 1);
+	g_sw.reverse = env_int("ANNI_REVERSE", 1, 0, 1);
+	g_sw.keep_mb = env_int("ANNI_KEEP_MB", 256, 0, 1 << 20);
+	g_sw.pipe = env_int("ANNI_PIPE", 1, 0, 2);
+	g_sw.tiles_per_wg = env_int("ANNI_TILES_PER_WG", -1, -1, 1 << 20);
+	g_sw.loaded = 1;
+}
+
+static const Switches &sw(void)
+{
+	if (!g_sw.loaded)
+		reload_switches();
+	return g_sw;
+}
+
 static int cu_count(void)
 {
 	static int cus;
@@ -1188,16 +1222,13 @@ static int cu_count(void)
 	return cus;
 }
 
-/* ANNI_BLOCKS_PER_CU: workgroups per compute unit of a grid that is resident as a whole (default 8). */
+/* A grid that is resident as a whole: ANNI_BLOCKS_PER_CU workgroups per compute unit (default 8). */
 int grid_for(int64_t n)
 {
-	static int per_cu;
 	int64_t tiles = (n + kTile - 1) / kTile;
 	int64_t g;
 
-	if (!per_cu)
-		per_cu = env_int("ANNI_BLOCKS_PER_CU", 8, 1, 32);
-	g = (int64_t)cu_count() * per_cu;
+	g = (int64_t)cu_count() * sw().blocks_per_cu;
 	if (g > kMaxPartials)
 		g = kMaxPartials;
 	if (g > tiles)
@@ -1207,34 +1238,19 @@ int grid_for(int64_t n)
 	return (int)g;
 }
 
-/* ANNI_NT=0 switches the streaming (non-temporal) cache hint off. */
 static bool nt_on(void)
 {
-	static int on = -1;
-
-	if (on < 0)
-		on = env_int("ANNI_NT", 1, 0, 1);
-	return on != 0;
+	return sw().nt != 0;
 }
 
-/* ANNI_REVERSE=0: the update walks the tiles from the first to the last. */
 static bool reverse_on(void)
 {
-	static int on = -1;
-
-	if (on < 0)
-		on = env_int("ANNI_REVERSE", 1, 0, 1);
-	return on != 0;
+	return sw().reverse != 0;
 }
 
-/* ANNI_KEEP_MB: how much of the gradients' tail the sum of squares leaves in the memory-side cache. */
 static int keep_mb(void)
 {
-	static int mb = -1;
-
-	if (mb < 0)
-		mb = env_int("ANNI_KEEP_MB", 256, 0, 1 << 20);
-	return mb;
+	return sw().keep_mb;
 }
 
 static bool aligned(const void *p, uintptr_t a)
@@ -1336,14 +1352,9 @@ int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *parti
 #define ANNI_UPDATE_UNROLL_NARROW 4	/* bf16 moments / bf16 or fp8 gradients */
 #endif
 
-/* ANNI_PIPE=0 keeps the narrow storage modes on the plain kernel, 2 pipelines the all-f32 mode too (for comparison). */
 static int pipe_level(void)
 {
-	static int on = -1;
-
-	if (on < 0)
-		on = env_int("ANNI_PIPE", 1, 0, 2);
-	return on;
+	return sw().pipe;
 }
 
 template <int GT, int MT>
@@ -1397,13 +1408,11 @@ static void update_launch(hipStream_t st, int grid, const UpdateArgs &a)
 */
 static int balanced_grid(int64_t n, int tiles_per_wg)
 {
-	static int per = -2;
 	const int64_t tiles = (n + kTile - 1) / kTile;
+	const int per = sw().tiles_per_wg;
 	int grid = grid_for(n);
 	int k;
 
-	if (per == -2)
-		per = env_int("ANNI_TILES_PER_WG", -1, -1, 1 << 20);
 	k = per >= 0 ? per : tiles_per_wg;
 	if (k > 0 && tiles / k > grid)
 		grid = (int)(tiles / k);

@@ -112,6 +112,7 @@ _PROTOS = {
     "anni_adam_enable_derived": (C.c_int, [C.POINTER(Adam), C.POINTER(Pack), C.c_int, C.c_int64]),
     "anni_adam_timed_derived_ms": (C.c_float, [C.POINTER(Adam)]),
     "anni_gpu_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int)]),
+    "anni_gpu_reload_switches": (None, []),
     "anni_lr_set_schedule": (None, [C.c_int, C.c_int, C.c_char_p]),
     "anni_lr_set_sched_from": (None, [C.c_int]),
     "anni_lr_step": (C.c_double, [C.c_double, C.c_int]),

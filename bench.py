@@ -76,6 +76,77 @@ def fill_grad_slots(L, opt, tensors, count, grad_type, seed, first_step=0):
     return ptrs, scales
 
 
+def sweep_leg(L, workload, spec, rounds=3, timed=6):
+    """One arena, one process, the values of one switch taking turns: per value the mean step,
+    sum-of-squares and update time (ms, HIP events) over rounds x timed steps.  Two processes
+    differ by the memory they were given by a per cent or two, more than most settings do; runs
+    inside one process repeat to about 0.1 %."""
+    from anni_amd import layout
+    from anni_amd.lm_adam import LmAdam
+    name, _, vals = spec.partition("=")
+    vals = [v for v in vals.split(",") if v != ""]
+    if not name.startswith("ANNI_") or not vals:
+        sys.exit("bench.py: --sweep wants NAME=V1,V2,... with an ANNI_* switch")
+    size, gt, mt, _nb, _ub = WORKLOADS[workload]
+    tensors = layout.tensors(size, "baseline")
+    slots = 8
+    opt = LmAdam(tensors, grad_type=gt, moment_type=mt, twins=True, skip_nonfinite=True,
+                 grad_slots=slots, beta2=0.95, weight_decay=0.1, grad_clip=1.0)
+    n = opt.n
+    assert L.anni_fill_normal_f32(opt.o.d_param, n, 20260101, 1, 0.0, 0.02) == 0
+    opt.seed_twins()
+    unit = 1.0 / (math.sqrt(n) * 1e-3)
+    step = 0
+    scales = []
+
+    def run(count):
+        nonlocal step
+        tot = [0.0, 0.0, 0.0]
+        for i in range(count):
+            k = (step + i) % slots
+            if gt == 2:
+                opt.o.d_gscale = scales[k].ptr
+            ms, sa, sb = C.c_float(0), C.c_float(0), C.c_float(0)
+            rc = L.anni_adam_time_steps(opt.h, 1, (C.c_void_p * 1)(ring[k]), 1,
+                                        C.byref(C.c_double(1e-4)),
+                                        C.byref(C.c_double(unit * (1.7 if (step + i) % 2 else 0.6))),
+                                        C.byref(ms), C.byref(sa), C.byref(sb))
+            assert rc == 0, L.gpu_debug_last_error()
+            tot = [tot[0] + ms.value, tot[1] + sa.value, tot[2] + sb.value]
+        step += count
+        return [t / count for t in tot]
+
+    old = os.environ.get(name)
+    res = {v: [] for v in vals}
+    try:
+        for _round in range(rounds):
+            for v in vals:
+                os.environ[name] = v
+                L.anni_gpu_reload_switches()
+                for sc in scales:
+                    if sc is not None:
+                        sc.free()
+                ring, scales = fill_grad_slots(L, opt, tensors, slots, gt, 20260101, step)
+                run(2)
+                res[v].append(run(timed))
+    finally:
+        if old is None:
+            os.environ.pop(name, None)
+        else:
+            os.environ[name] = old
+        L.anni_gpu_reload_switches()
+    out = {"workload": workload, "switch": name, "placement_probe_GBps": round(opt.probe_gbps, 1),
+           "rounds": rounds, "timed_steps_per_round": timed, "values": {}}
+    for v in vals:
+        r = res[v]
+        out["values"][v] = {"step_ms": round(sum(x[0] for x in r) / len(r), 4),
+                            "sumsq_ms": round(sum(x[1] for x in r) / len(r), 4),
+                            "update_ms": round(sum(x[2] for x in r) / len(r), 4),
+                            "update_ms_rounds": [round(x[2], 4) for x in r]}
+    opt.free()
+    return out
+
+
 def cpu_baselines(size_name, norm_bpp, upd_bpp, budget_s):
     """The step on the host cores of this box: (multithreaded port, single-thread reference)."""
     from anni_amd import layout
@@ -358,6 +429,10 @@ def main():
                     choices=["both", "fp8", "pack"],
                     help="the reference's own tensor list (separate Wq, Wk, Wv) with the fused "
                          "producers on: E4M3 twins of every matrix and a packed [Wq|Wk|Wv] per block")
+    ap.add_argument("--sweep", default=None, metavar="NAME=V1,V2,...",
+                    help="time the step under each value of one tuning switch (ANNI_TILES_PER_WG, "
+                         "ANNI_KEEP_MB, ANNI_REVERSE, ANNI_PIPE, ANNI_NT, ANNI_BLOCKS_PER_CU) on ONE "
+                         "arena in this process, the settings taking turns (one JSON line)")
     ap.add_argument("--ref-jsonl", default=None, metavar="FILE",
                     help="also append one row in the reference's bench-log schema (optimizer "
                          "phase only); steps are then timed one call each")
@@ -391,6 +466,9 @@ def main():
         return
     if a.reference_caller_only:
         print(json.dumps(reference_caller_leg(L)))
+        return
+    if a.sweep:
+        print(json.dumps({"sweep": sweep_leg(L, a.workload, a.sweep)}))
         return
 
     size, gt, mt, norm_bpp, upd_bpp = WORKLOADS[a.workload]

@@ -194,6 +194,14 @@ double	anni_lr_step(double base_lr, int step);
 void	*anni_gpu_stream(void);
 void	anni_gpu_set_stream(void *hip_stream);
 
+/*
+** Reads the kernels' tuning switches (ANNI_TILES_PER_WG, ANNI_KEEP_MB, ANNI_REVERSE, ANNI_PIPE,
+** ANNI_NT, ANNI_BLOCKS_PER_CU) from the environment again; without this call they are read once,
+** on first use.  For sweeps that compare settings on one arena inside one process
+** (`bench.py --sweep`); results never depend on them.  No counterpart in the reference.
+*/
+void	anni_gpu_reload_switches(void);
+
 /* Name and architecture of the current device and the HIP driver version: what the reference's bench row records from nvidia-smi (lang/lm_bench.c:287-316). */
 int	anni_gpu_device_info(char *name, size_t cap, int *driver_version);
 

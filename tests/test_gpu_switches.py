@@ -1,7 +1,7 @@
 """The tile walk and cache-hint switches of the step change where data is found, never a bit:
 sum of squares (two loops, changeover at any tile), update walking forward or backward, with
 non-temporal hints or without.  Each setting runs in a process of its own (the library reads its
-switches once), and all settings that share a grid must print the same digests."""
+switches once unless told to read them again), and all settings that share a grid must print the same digests."""
 import json
 import os
 import subprocess
