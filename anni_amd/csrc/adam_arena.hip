@@ -302,10 +302,10 @@ static anni_adam *create_body(const anni_tensor *tensors, int n_tensors,
 	const size_t big = (size_t)2 << 20;	/* each flat starts on a 2 MiB boundary */
 	/* Spread arenas auditioned at most (a second one while the first stays below these figures). */
 	const int kTries = 2;
-	/* (good placements measure 6390-6480 / 6180-6320 / 6380-6430 in the three cases; others come 3 - 8 % lower) */
-	const double kGoodGBps = 6250.0;		/* all-f32 storage */
-	const double kGoodGBpsBf16 = 6100.0;		/* bf16 moments */
-	const double kGoodGBpsNarrow = 6250.0;		/* f32 moments, bf16 or fp8 gradients */
+	/* (good placements measure 6450-6570 / 6400-6460 / 6430-6520 in the three cases; others come 2 - 5 % lower) */
+	const double kGoodGBps = 6400.0;		/* all-f32 storage */
+	const double kGoodGBpsBf16 = 6350.0;		/* bf16 moments */
+	const double kGoodGBpsNarrow = 6400.0;		/* f32 moments, bf16 or fp8 gradients */
 	anni_adam *opt;
 	anni_adam_priv *pv;
 	Sizes z;
