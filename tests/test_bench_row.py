@@ -76,3 +76,17 @@ def test_rows_of_two_runs_match_and_never_match_a_whole_step_row(tmp_path):
 
 def test_strings_are_made_json_safe():
     assert bench_row._json_safe('a"b\\c\n') == "a_b_c_"
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """One GPU is all this build runs on: a larger --gpus ends with a message that says so,
+    before any device or library is touched."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in r.stderr and "--gpus 1" in r.stderr
+    assert r.stdout.strip() == ""
