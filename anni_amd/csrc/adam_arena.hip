@@ -53,6 +53,8 @@ struct anni_adam_priv {
 	float			*d_tile_amax;	/* per-wavefront max |p| of every whole tile */
 	int			fp8_twins;	/* 1: some tensor keeps an E4M3 twin */
 	float			der_ms;		/* E4M3 pass time summed by anni_adam_time_steps */
+	/* scratch of anni_adam_quantize_grads, allocated at its first call: per-tensor max words, then the tile maxima */
+	void			*gq_scratch;
 };
 
 static size_t elem_bytes(int type)
@@ -496,6 +498,8 @@ void anni_adam_free(anni_adam **popt)
 			(void)hip_ok(hipFree(opt->priv->arena), "arena hipFree");
 		if (opt->priv->derived && opt->priv->derived_owned)
 			(void)hip_ok(hipFree(opt->priv->derived), "derived hipFree");
+		if (opt->priv->gq_scratch)
+			(void)hip_ok(hipFree(opt->priv->gq_scratch), "quantizer hipFree");
 		if (opt->priv->h_state)
 			(void)hip_ok(hipHostFree(opt->priv->h_state), "arena hipHostFree");
 		delete opt->priv;
@@ -680,6 +684,52 @@ int anni_adam_zero_grad(anni_adam *opt)
 		return -1;
 	return launch_fill_bytes(compute_stream(), opt->d_grad, 0,
 	    (size_t)opt->n * elem_bytes(opt->cfg.grad_type));
+}
+
+int anni_adam_quantize_grads(anni_adam *opt, const float *d_src)
+{
+	anni_adam_priv *pv;
+	hipStream_t st;
+	Flat f;
+	size_t amax_bytes;
+
+	if (!opt || !opt->priv || !d_src || !opt->d_grad || !opt->d_gscale || !device_ready()
+	    || opt->cfg.grad_type != ANNI_FP8_E4M3 || ((uintptr_t)d_src & 15) != 0)
+		return -1;
+	pv = opt->priv;
+	st = compute_stream();
+	amax_bytes = round_up((size_t)opt->n_tensors * sizeof(uint32_t), 256);
+	if (!pv->gq_scratch) {
+		const size_t n_tiles = (size_t)((opt->n + kTile - 1) / kTile);
+		void *d = nullptr;
+
+		if (!hip_ok(hipMalloc(&d, amax_bytes + n_tiles * kWaves * sizeof(float)),
+		    "quantizer hipMalloc")) {
+			(void)hipGetLastError();
+			return -1;
+		}
+		pv->gq_scratch = d;
+	}
+	/*
+	** The passes that keep the E4M3 weight twins, pointed at the gradients and at every tensor:
+	** maxima of whole tiles per wavefront (tiles shared by tensors raise the tensors' words
+	** directly), folded into one word per tensor, then scale_t = max(amax_t / 448, 1e-12) and
+	** q = E4M3(x * (1 / scale_t)) -- the arithmetic of anni_fp8_quantize on each tensor.
+	*/
+	memset(&f, 0, sizeof(f));
+	f.p = const_cast<float *>(d_src);
+	f.n = opt->n;
+	f.segs = pv->d_segs;
+	f.tile_seg = pv->d_tile_seg;
+	f.der.wamax = (uint32_t *)pv->gq_scratch;
+	f.der.tile_amax = (float *)((char *)pv->gq_scratch + amax_bytes);
+	if (launch_fill_bytes(st, f.der.wamax, 0, (size_t)opt->n_tensors * sizeof(uint32_t)) != 0
+	    || launch_derive(st, f, 0u) != 0
+	    || launch_amax_fold(st, f, nullptr, 0u) != 0
+	    || launch_fp8_twins(st, f, (uint8_t *)opt->d_grad, opt->d_gscale, f.der.wamax,
+	    opt->n_tensors, nullptr, 0u) != 0)
+		return -1;
+	return 0;
 }
 
 } /* extern "C" */

@@ -138,20 +138,22 @@ int	launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double gra
 ** Derived outputs straight from p, without an update (after weights were loaded):
 ** wamax and the packed matrices as the update would leave them.
 */
-int	launch_derive(hipStream_t st, const Flat &f);
+int	launch_derive(hipStream_t st, const Flat &f, uint32_t need = kSegFp8Twin);
 /*
 ** wamax[s] = max(wamax[s], tile maxima of tensor s) for the flagged tensors, after
 ** launch_update or launch_derive on the same stream.  state (may be NULL): nothing to do
 ** after a skipped step.
 */
-int	launch_amax_fold(hipStream_t st, const Flat &f, const StepState *state);
+int	launch_amax_fold(hipStream_t st, const Flat &f, const StepState *state,
+		uint32_t need = kSegFp8Twin);
 /*
-** q = E4M3(p * (1 / scale_s)) for the tensors flagged kSegFp8Twin, scale_s from wamax[s]
-** (num/gpu_cuda.cu:826-851,927-938); wscale[s] receives the scale.  state (may be NULL): a
-** skipped step leaves q and wscale alone.
+** q = E4M3(p * (1 / scale_s)) for the tensors flagged `need` (0: every tensor), scale_s from
+** wamax[s] (num/gpu_cuda.cu:826-851,927-938); wscale[s] receives the scale.  state (may be
+** NULL): a skipped step leaves q and wscale alone.
 */
 int	launch_fp8_twins(hipStream_t st, const Flat &f, uint8_t *q, float *wscale,
-		const uint32_t *wamax, int n_tensors, const StepState *state);
+		const uint32_t *wamax, int n_tensors, const StepState *state,
+		uint32_t need = kSegFp8Twin);
 int	launch_f32_to_bf16(hipStream_t st, uint16_t *dst, const float *src, int64_t n);
 /* pairs[2k] = m[first+k], pairs[2k+1] = v[first+k] as floats (bf16 moments widen exactly). */
 int	launch_mv_interleave(hipStream_t st, float *pairs, const void *m, const void *v,

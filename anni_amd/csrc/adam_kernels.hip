@@ -899,7 +899,14 @@ struct DeriveArgs {
 	const int32_t	*tile_seg;
 	Derived		der;
 	int		vec_ok;
+	uint32_t	need;	/* tensors whose max |x| is wanted: those with this flag; 0 = every tensor */
 };
+
+/* Does a tensor with these flags take part, given the flag a pass asks for (0 = every tensor)? */
+__device__ __forceinline__ bool wanted(uint32_t flags, uint32_t need)
+{
+	return need == 0u || (flags & need) != 0u;
+}
 
 template <bool NT>
 __global__ __launch_bounds__(kThreads) void derive_kernel(DeriveArgs a)
@@ -914,7 +921,7 @@ __global__ __launch_bounds__(kThreads) void derive_kernel(DeriveArgs a)
 
 		if (a.vec_ok && end - base == kTile && a.segs[s].end >= end) {
 			const uint32_t flags = a.segs[s].flags;
-			const bool fp8w = (flags & kSegFp8Twin) != 0 && a.der.wamax != nullptr;
+			const bool fp8w = wanted(flags, a.need) && a.der.wamax != nullptr;
 			const bool pk = (flags & kSegPack) != 0 && a.der.pack != nullptr;
 			float amax_l = 0.0f;
 
@@ -945,7 +952,7 @@ __global__ __launch_bounds__(kThreads) void derive_kernel(DeriveArgs a)
 				const uint32_t flags = a.segs[s].flags;
 				const float x = a.p[i];
 
-				if ((flags & kSegFp8Twin) != 0 && a.der.wamax != nullptr) {
+				if (wanted(flags, a.need) && a.der.wamax != nullptr) {
 					const float ab = fmaxf(0.0f, fabsf(x));
 
 					if (ab > 0.0f)
@@ -965,6 +972,7 @@ struct FoldArgs {
 	const float	*tile_amax;
 	uint32_t	*wamax;
 	const StepState	*state;
+	uint32_t	need;
 };
 
 /*
@@ -986,7 +994,7 @@ __global__ __launch_bounds__(kThreads) void amax_fold_kernel(FoldArgs a)
 		const int64_t base = tile * kTile;
 
 		if (base + kTile <= a.n && a.segs[t].end >= base + kTile
-		    && (a.segs[t].flags & kSegFp8Twin) != 0) {
+		    && wanted(a.segs[t].flags, a.need)) {
 			const f32x4 w = *(const f32x4 *)(a.tile_amax + tile * kWaves);
 
 			s = t;
@@ -1017,6 +1025,7 @@ struct Fp8TwinArgs {
 	int		n_tensors;
 	const StepState	*state;
 	int		vec_ok;
+	uint32_t	need;
 };
 
 /*
@@ -1034,7 +1043,7 @@ __global__ __launch_bounds__(kThreads) void fp8_twin_kernel(Fp8TwinArgs a)
 
 	if (blockIdx.x == 0) {
 		for (int s = tid; s < a.n_tensors; s += kThreads) {
-			if (!skipped && (a.segs[s].flags & kSegFp8Twin) != 0)
+			if (!skipped && wanted(a.segs[s].flags, a.need))
 				a.wscale[s] = scale_from_amax(__uint_as_float(a.wamax[s]));
 		}
 	}
@@ -1046,7 +1055,7 @@ __global__ __launch_bounds__(kThreads) void fp8_twin_kernel(Fp8TwinArgs a)
 		int s = a.tile_seg[tile];
 
 		if (a.vec_ok && end - base == kTile && a.segs[s].end >= end) {
-			if ((a.segs[s].flags & kSegFp8Twin) == 0)
+			if (!wanted(a.segs[s].flags, a.need))
 				continue;
 			const float inv = 1.0f / scale_from_amax(__uint_as_float(a.wamax[s]));
 			f32x4 P[kQuadsPerTile];
@@ -1065,7 +1074,7 @@ __global__ __launch_bounds__(kThreads) void fp8_twin_kernel(Fp8TwinArgs a)
 			for (int64_t i = base + tid; i < end; i += kThreads) {
 				while (i >= a.segs[s].end)
 					s++;
-				if ((a.segs[s].flags & kSegFp8Twin) != 0) {
+				if (wanted(a.segs[s].flags, a.need)) {
 					const float inv = 1.0f / scale_from_amax(__uint_as_float(a.wamax[s]));
 
 					a.q[i] = (uint8_t)fp8_e4m3_encode(a.p[i] * inv);
@@ -1504,7 +1513,7 @@ int launch_f32_to_bf16(hipStream_t st, uint16_t *dst, const float *src, int64_t 
 	return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
-int launch_derive(hipStream_t st, const Flat &f)
+int launch_derive(hipStream_t st, const Flat &f, uint32_t need)
 {
 	DeriveArgs a;
 
@@ -1515,6 +1524,7 @@ int launch_derive(hipStream_t st, const Flat &f)
 	a.segs = f.segs;
 	a.tile_seg = f.tile_seg;
 	a.der = f.der;
+	a.need = need;
 	a.vec_ok = aligned(f.p, 16) ? 1 : 0;
 	if (f.der.wamax && !a.vec_ok)
 		return -1;
@@ -1525,7 +1535,7 @@ int launch_derive(hipStream_t st, const Flat &f)
 	return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
-int launch_amax_fold(hipStream_t st, const Flat &f, const StepState *state)
+int launch_amax_fold(hipStream_t st, const Flat &f, const StepState *state, uint32_t need)
 {
 	FoldArgs a;
 	const int64_t n_tiles = (f.n + kTile - 1) / kTile;
@@ -1539,13 +1549,14 @@ int launch_amax_fold(hipStream_t st, const Flat &f, const StepState *state)
 	a.tile_amax = f.der.tile_amax;
 	a.wamax = f.der.wamax;
 	a.state = state;
+	a.need = need;
 	hipLaunchKernelGGL(amax_fold_kernel, dim3((unsigned)((n_tiles + kThreads - 1) / kThreads)),
 	    dim3(kThreads), 0, st, a);
 	return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
 int launch_fp8_twins(hipStream_t st, const Flat &f, uint8_t *q, float *wscale,
-	const uint32_t *wamax, int n_tensors, const StepState *state)
+	const uint32_t *wamax, int n_tensors, const StepState *state, uint32_t need)
 {
 	Fp8TwinArgs a;
 
@@ -1561,6 +1572,7 @@ int launch_fp8_twins(hipStream_t st, const Flat &f, uint8_t *q, float *wscale,
 	a.wscale = wscale;
 	a.n_tensors = n_tensors;
 	a.state = state;
+	a.need = need;
 	a.vec_ok = aligned(f.p, 16) && aligned(q, 4) ? 1 : 0;
 	if (nt_on())
 		hipLaunchKernelGGL((fp8_twin_kernel<true>), dim3(balanced_grid(f.n, 1)), dim3(kThreads), 0, st, a);

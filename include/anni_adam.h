@@ -155,6 +155,16 @@ int	anni_adam_seed_twins(anni_adam *opt);
 /* lm_adam_zero_grad: clears the gradient flat on the stream. */
 int	anni_adam_zero_grad(anni_adam *opt);
 /*
+** The producer side of the fp8 gradient format (grad_type ANNI_FP8_E4M3): d_src, a device flat
+** of n floats in the optimizer's tensor order (16-byte aligned), is quantised into the bound
+** gradient flat and d_gscale, every tensor with its own scale = max(max|x| / 448, 1e-12) and
+** q = E4M3(x * (1 / scale)), saturating -- the arithmetic of anni_fp8_quantize and of the
+** reference's FP8 quantiser (num/gpu_cuda.cu:826-851,927-938) on each tensor, in four launches
+** for the whole flat instead of four per tensor.  Asynchronous on the compute stream; allocates
+** its scratch at the first call.  No counterpart in the reference (it has no fp8 gradients).
+*/
+int	anni_adam_quantize_grads(anni_adam *opt, const float *d_src);
+/*
 ** lm_adam_step_scaled (lm_adam.c:522-607): lr <= 0 returns 1 without advancing t;
 ** otherwise t++, [sum of squares when grad_clip > 0 or skip_nonfinite], update.
 ** Asynchronous on the compute stream: nothing is read back.

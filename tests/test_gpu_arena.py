@@ -306,6 +306,62 @@ def test_fp8_gradients_with_per_tensor_scale_and_skip(gpu, oracle):
     opt.free()
 
 
+def test_multi_tensor_gradient_quantiser_equals_the_per_tensor_one(gpu, oracle):
+    """anni_adam_quantize_grads: the whole float gradient flat into E4M3 codes and per-tensor scales
+    in four launches -- identical, code for code and scale for scale, to the oracle's quantiser on
+    each tensor (which the per-tensor device quantiser equals): tensors that share tiles, single
+    elements, an all-zero tensor, values up to the saturation point, a NaN, and a step after it."""
+    from anni_amd.lm_adam import DeviceBuffer
+    rng = np.random.default_rng(808)
+    tensors = [(6000, 3), (64, 0), (4096, 3), (8192 + 3, 3), (1, 0), (20000, 3), (3, 0),
+               (4096 * 5, 3), (777, 1), (2, 0)]
+    opt = make(gpu, tensors, grad_type=FP8, beta2=0.95, weight_decay=0.1, grad_clip=1.0,
+               skip_nonfinite=True)
+    n = opt.n
+    p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    opt.upload("param", p0)
+    opt.seed_twins()
+    src = DeviceBuffer(n * 4)
+    for case in range(3):
+        g32 = (rng.standard_normal(n) * 10.0 ** rng.integers(-6, 2, n)).astype(np.float32)
+        for i, (off, cnt) in enumerate(zip(opt.offsets, opt.sizes)):
+            g32[off:off + cnt] *= np.float32(1.0 + 3 * i)
+        o2, c2 = opt.offsets[2], opt.sizes[2]
+        g32[o2:o2 + c2] = 0.0                                  # amax 0: scale 1e-12, codes 0
+        g32[opt.offsets[6]] = -0.0
+        if case == 1:
+            g32[opt.offsets[3] + 4100] = np.nan                # the NaN becomes the NaN code
+        src.upload(g32)
+        assert gpu.anni_adam_quantize_grads(opt.h, src.ptr) == 0
+        assert gpu.gpu_stream_sync() == 0
+        q = opt.download("grad")
+        sc = opt.download("gscale")
+        for i, (off, cnt) in enumerate(zip(opt.offsets, opt.sizes)):
+            qw, sw = oracle.fp8_quantize(g32[off:off + cnt])
+            assert (q[off:off + cnt] == qw).all(), (case, i)
+            assert np.float32(sc[i]).view(np.uint32) == np.float32(sw).view(np.uint32), (case, i)
+        # and the step takes them: skipped with the NaN, bit for bit otherwise
+        P, M, V = opt.download("param"), opt.download("m"), opt.download("v")
+        t0 = opt.t
+        opt.step_scaled(1e-3)
+        st = opt.sync_stats()
+        assert st.last_skipped == (1 if case == 1 else 0)
+        O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True,
+                          grad_type=oracle.FP8, tensors=oracle_tensors(opt, sc), threads=4)
+        O.o.t = t0
+        O.step(P, q.copy(), M, V, 1e-3, sumsq_override=None if case == 1 else st.last_sumsq)
+        assert same_bits(opt.download("param"), P) and same_bits(opt.download("m"), M)
+        assert same_bits(opt.download("v"), V)
+    # refusals: not an fp8 arena, no source, unaligned source
+    assert gpu.anni_adam_quantize_grads(opt.h, None) == -1
+    assert gpu.anni_adam_quantize_grads(opt.h, src.ptr + 4) == -1
+    other = make(gpu, [(100, 0)])
+    assert gpu.anni_adam_quantize_grads(other.h, src.ptr) == -1
+    other.free()
+    src.free()
+    opt.free()
+
+
 def test_fp8_decode_all_codes_on_device(gpu, oracle):
     """Every E4M3 byte through the kernel's decoder: with m = v = 0 and t = 1, m = (1-b1) * g."""
     opt = make(gpu, [(256, 0)], grad_type=FP8, beta1=0.5, beta2=0.5)
