@@ -40,7 +40,7 @@ ELEM = {0: 4, 1: 2, 2: 1}
 # HBM bytes per launch of the update kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled
 # by what the counter reads for a plain copy kernel of known size (summaries under profiles/).
 TRAFFIC_BYTES = {"555m": 18907053045, "185m": 5712778091, "555m-bf16": 12236824127,
-                 "1p4b-fp8": 39598974009}
+                 "1p4b-fp8": 39599067321}
 STORAGE = {"185m": "f32 p/g/m/v + bf16 twin", "555m": "f32 p/g/m/v + bf16 twin",
            "555m-bf16": "f32 p, bf16 g/m/v + bf16 twin",
            "1p4b-fp8": "f32 p/m/v, fp8-e4m3 g with per-tensor scale + bf16 twin",
