@@ -1423,8 +1423,11 @@ static int balanced_grid(int64_t n, int tiles_per_wg)
 	int k;
 
 	k = per >= 0 ? per : tiles_per_wg;
-	if (k > 0 && tiles / k > grid)
-		grid = (int)(tiles / k);
+	if (k > 0 && tiles / k > grid) {
+		const int64_t cap = (int64_t)1 << 22;	/* 2^30 lanes: within every launch limit; more tiles than that take turns */
+
+		grid = (int)(tiles / k < cap ? tiles / k : cap);
+	}
 	return grid;
 }
 
