@@ -917,10 +917,19 @@ __global__ __launch_bounds__(kThreads) void derive_kernel(DeriveArgs a)
 	for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
 		const int64_t base = tile * kTile;
 		const int64_t end = base + kTile < a.n ? base + kTile : a.n;
-		int s = a.tile_seg[tile];
+		const bool whole = a.vec_ok && end - base == kTile;
+		f32x4 P[kQuadsPerTile] = {};
 
-		if (a.vec_ok && end - base == kTile && a.segs[s].end >= end) {
-			const uint32_t flags = a.segs[s].flags;
+		/* a whole tile's loads go out before the launch table is asked whose tile it is */
+		if (whole) {
+#pragma unroll
+			for (int u = 0; u < kQuadsPerTile; u++)
+				P[u] = load_quad<kF32, NT>(a.p, base + (int64_t)(u * kThreads + tid) * kQuad, 1.0f);
+		}
+		int s = table(a.tile_seg)[tile];
+
+		if (whole && table(a.segs)[s].end >= end) {
+			const uint32_t flags = table(a.segs)[s].flags;
 			const bool fp8w = wanted(flags, a.need) && a.der.wamax != nullptr;
 			const bool pk = (flags & kSegPack) != 0 && a.der.pack != nullptr;
 			float amax_l = 0.0f;
@@ -928,17 +937,16 @@ __global__ __launch_bounds__(kThreads) void derive_kernel(DeriveArgs a)
 			if (!fp8w && !pk)
 				continue;
 			const PackDesc pd = pk ? a.der.packs[s] : PackDesc{0, 1u, 0u};
-			const int64_t seg_begin = a.segs[s].begin;
+			const int64_t seg_begin = table(a.segs)[s].begin;
 
 #pragma unroll
 			for (int u = 0; u < kQuadsPerTile; u++) {
 				const int64_t idx = base + (int64_t)(u * kThreads + tid) * kQuad;
-				const f32x4 P = load_quad<kF32, NT>(a.p, idx, 1.0f);
 
 				if (fp8w)
-					amax_l = amax4(amax_l, P);
+					amax_l = amax4(amax_l, P[u]);
 				if (pk)
-					pack_quad<NT>(a.der.pack, pd, (uint32_t)(idx - seg_begin), P);
+					pack_quad<NT>(a.der.pack, pd, (uint32_t)(idx - seg_begin), P[u]);
 			}
 			if (fp8w) {
 				amax_l = wave_max(amax_l);
