@@ -20,13 +20,19 @@
 **                                  (bias / LayerNorm gradients as serial float column sums)
 **
 ** Pinned by: the reference's compiled lm_adam_step_scaled (oracle/_ref, bit for
-** bit on p/m/v), the reference's own LR known answers (tests/test_ann.c:866-879),
-** closed forms (t=1, constant gradient, zero gradient), and brute-force
-** long-double sums; oracle_colsum_add by the reference's compiled layernorm_backward
-** (dgamma / dbeta, bit for bit) and by inputs whose sum depends on the order.  PARITY UNPINNED by the reference (no implementation exists
-** there, the oracle defines them): bf16-stored m/v, bf16 gradients, fp8-E4M3
-** gradients with a per-tensor scale, weight decay on selected tensors only, and
-** the non-finite skip on the CPU path.
+** bit on p/m/v), the golden vectors it wrote (tests/golden/*.npz: oracle_adam_step_scaled
+** and oracle_adam_step_slots, bit for bit), the reference's own LR known answers
+** (tests/test_ann.c:866-879), closed forms (t=1, constant gradient, zero gradient), and
+** brute-force exact sums; oracle_colsum_add by the reference's compiled layernorm_backward
+** (dgamma / dbeta, bit for bit) and by inputs whose sum depends on the order.  The VALUE of
+** the FP8 norm (oracle_sumsq's factored form) is pinned against the direct form
+** SUM (float(decode(q) * scale_t) * grad_scale)^2 summed exactly (<= 1e-7 relative, multi-tensor
+** lists) and by invariants a wrong factoring fails (a tensor's share scales with the square
+** of its own scale only, one element gives the closed form, permutations inside a tensor
+** change no bit, a NaN code gives NaN).
+** PARITY UNPINNED by the reference (no implementation exists there, the oracle defines the
+** rounding points): bf16-stored m/v, bf16 gradients, fp8-E4M3 gradients with a per-tensor
+** scale, weight decay on selected tensors only, and the non-finite skip on the CPU path.
 */
 #ifndef ADAM_ORACLE_H__
 #define ADAM_ORACLE_H__
@@ -87,7 +93,8 @@ int	oracle_adam_step_scaled(oracle_adam *o, float *p, void *g, void *m, void *v,
 
 /*
 ** Sum over the flat of (g*grad_scale)^2 as the clip block computes it.  FP8 gradients use the
-** factored form SUM_t (scale_t*grad_scale)^2 * SUM_i decode(q_i)^2 (defined here, unpinned).
+** factored form SUM_t (scale_t*grad_scale)^2 * SUM_i decode(q_i)^2 (within 1e-7 relative of the
+** direct form the update consumes; tests/test_oracle.py).
 */
 double	oracle_sumsq(const void *g, int grad_type, int64_t n, const oracle_seg *segs,
 		int nsegs, double grad_scale, int threads);

@@ -363,6 +363,108 @@ def test_storage_modes_round_where_documented(oracle):
     assert same_bits(p_c, p_d) and same_bits(m_c, m_d) and same_bits(v_c, v_d) and not qq.any()
 
 
+# ---- the FP8 norm's value and the slot-layout loop (the last two functions nothing pinned) ----
+
+def _fp8_direct_sumsq(q, tensors, gs, table):
+    """Brute force of what the update consumes: g_i = float32(decode(q_i) * scale_t), then
+    (double(g_i) * gs)^2 summed exactly."""
+    terms = []
+    for off, cnt, _wd, sc in tensors:
+        g = (table[q[off:off + cnt]] * np.float32(sc)).astype(np.float32)
+        terms.extend((float(x) * gs) ** 2 for x in g)
+    return math.fsum(terms)
+
+
+def _fp8_case(rng, sizes):
+    tensors, off = [], 0
+    for cnt in sizes:
+        tensors.append([off, cnt, 1, float(np.float32(rng.uniform(1e-6, 3e-3)))])
+        off += cnt
+    q = rng.integers(0, 256, off).astype(np.uint8)
+    q[(q & 0x7f) == 0x7f] = 0x3a                    # no NaN codes in the value test
+    return q, tensors
+
+
+@pytest.mark.parametrize("sizes", [
+    [5000, 1, 3000, 4096, 777],                     # tensors sharing a 4096-element tile, one element
+    [1, 1, 1], [4096, 4096], [8191, 3, 12289]])
+def test_fp8_sumsq_value_against_brute_force(oracle, sizes):
+    """oracle_sumsq's FP8 branch (the factored form) against the direct form, <= 1e-7 relative."""
+    rng = np.random.default_rng(sum(sizes))
+    table = oracle.fp8_decode_table()
+    q, tensors = _fp8_case(rng, sizes)
+    if len(sizes) == 5:
+        q[tensors[2][0]:tensors[2][0] + tensors[2][1]] = 0      # an all-zero tensor
+    for gs in (1.0, 0.37, 1 / 252.0):
+        want = _fp8_direct_sumsq(q, tensors, gs, table)
+        for threads in (1, 4):
+            got = oracle.sumsq(q, oracle.FP8, [tuple(t) for t in tensors], gs, threads)
+            assert abs(got - want) <= 1e-7 * want, (sizes, gs, threads, got, want)
+
+
+def test_fp8_sumsq_invariants(oracle):
+    """What a wrong factoring breaks: a tensor's share scales with the square of ITS scale only,
+    one element gives the closed form, the order of codes inside a tensor is irrelevant."""
+    rng = np.random.default_rng(11)
+    table = oracle.fp8_decode_table()
+    q, tensors = _fp8_case(rng, [3000, 500, 4096])
+    T = [tuple(t) for t in tensors]
+    base = oracle.sumsq(q, oracle.FP8, T, 0.5)
+    # share of tensor 1 alone (the other scales zeroed: exact zeros)
+    only1 = [(o, c, w, sc if i == 1 else 0.0) for i, (o, c, w, sc) in enumerate(T)]
+    share1 = oracle.sumsq(q, oracle.FP8, only1, 0.5)
+    rest = [(o, c, w, 0.0 if i == 1 else sc) for i, (o, c, w, sc) in enumerate(T)]
+    share_rest = oracle.sumsq(q, oracle.FP8, rest, 0.5)
+    assert abs(base - (share1 + share_rest)) <= 4e-16 * base
+    doubled = [(o, c, w, sc * 2 if i == 1 else sc) for i, (o, c, w, sc) in enumerate(T)]
+    got = oracle.sumsq(q, oracle.FP8, doubled, 0.5)
+    assert abs(got - (4.0 * share1 + share_rest)) <= 4e-16 * got        # x2 is exact, so is x4
+    # one element: (decode(q) * scale * gs)^2 up to the two roundings of the factored product
+    for code in (0x01, 0x38, 0x7e, 0xc5):
+        one = np.array([code], np.uint8)
+        sc = float(np.float32(7.25e-4))
+        want = (float(table[code]) * sc * 0.37) ** 2
+        got = oracle.sumsq(one, oracle.FP8, [(0, 1, 1, sc)], 0.37)
+        assert abs(got - want) <= 1e-15 * want
+    # permuting the codes inside each tensor changes nothing, bit for bit
+    qp = q.copy()
+    for o, c, _w, _s in T:
+        qp[o:o + c] = rng.permutation(qp[o:o + c])
+    assert oracle.sumsq(qp, oracle.FP8, T, 0.5) == base
+    # a NaN code anywhere makes the sum NaN (the skip decision of the step rests on it)
+    qn = q.copy()
+    qn[3100] = 0x7f
+    assert math.isnan(oracle.sumsq(qn, oracle.FP8, T, 0.5))
+
+
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+def test_slot_loop_matches_golden(oracle, name):
+    """oracle_adam_step_slots (the reference's 24-byte-slot layout, the serial timing leg of the
+    bench) bit for bit against the vectors the compiled reference wrote."""
+    import ctypes as C
+    G = load_golden(name)
+    n = G["p0"].size
+    p = G["p0"].copy()
+    g = np.zeros(n, np.float32)
+    slots = np.zeros(n, dtype=[("param", np.uint64), ("grad", np.uint64), ("m", np.float32),
+                               ("v", np.float32)])
+    assert slots.itemsize == 24
+    slots["param"] = p.ctypes.data + 4 * np.arange(n, dtype=np.uint64)
+    slots["grad"] = g.ctypes.data + 4 * np.arange(n, dtype=np.uint64)
+    L = oracle.lib()
+    L.oracle_adam_step_slots.argtypes = [C.c_void_p, C.c_int64, C.c_int] + [C.c_double] * 7
+    L.oracle_adam_step_slots.restype = None
+    for s in range(G["grads"].shape[0]):
+        g[:] = G["grads"][s]
+        L.oracle_adam_step_slots(slots.ctypes.data, n, s + 1, float(G["beta1"]), float(G["beta2"]),
+                                 float(G["eps"]), float(G["wd"]), float(G["clip"]),
+                                 float(G["lr"][s]), float(G["grad_scale"]))
+        assert same_bits(p, G["p"][s]), (name, s)
+        assert same_bits(np.ascontiguousarray(slots["m"]), G["m"][s])
+        assert same_bits(np.ascontiguousarray(slots["v"]), G["v"][s])
+        assert not g.any()
+
+
 # ---- bias / LayerNorm gradient column sums ---------------------------------------------------
 
 def test_colsum_matches_golden_of_the_reference(oracle):
