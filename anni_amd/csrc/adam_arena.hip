@@ -17,6 +17,7 @@
 #include "anni_adam.h"
 #include "anni_gpu.h"
 #include "backend_state.h"
+#include "placement.h"
 
 using namespace anni;
 
@@ -24,8 +25,11 @@ using namespace anni;
 static const size_t kStateBytes = 128 + ((kTicketBytes + 255) / 256) * 256;
 
 struct anni_adam_priv {
-	void			*arena;
-	size_t			arena_bytes;
+	void			*arena;		/* p, m and the tables (split), or everything (compact) */
+	void			*arena2;	/* split: v, the twins and the gradient slots */
+	size_t			arena_bytes;	/* both allocations together */
+	size_t			resident_bytes;	/* what a step touches: p, m, v, twins, one gradient flat, the tables */
+	double			apart_ratio;	/* split: time(all flats in one block) / time(this placement) on the probe */
 	Seg			*d_segs;
 	int32_t			*d_tile_seg;
 	double			*d_partials;
@@ -34,17 +38,11 @@ struct anni_adam_priv {
 	char			*grad_slots;	/* the arena's gradient flats (NULL when external) */
 	size_t			grad_slot_bytes;	/* distance between consecutive slots */
 	int			n_grad_slots;
-	int			spread;		/* 1: every flat in its own region of device memory */
+	int			split;		/* 1: two allocations (see the layout note in anni_adam_create) */
 	double			probe_gbps;	/* update throughput measured at creation (0: not measured) */
 	std::vector<int64_t>	offsets;
 	std::vector<uint32_t>	flags;
-	char			*hole;		/* spread: unused rest of the tables' region (NULL: none) */
-	size_t			hole_bytes;
-	/*
-	** derived outputs (anni_adam_enable_derived): in the hole of a spread arena, which
-	** keeps them a region away from p, m, v, the twins and the gradients; else one more
-	** allocation
-	*/
+	/* derived outputs (anni_adam_enable_derived): one more allocation */
 	std::vector<Seg>	segs;		/* host copy of the device table */
 	void			*derived;
 	int			derived_owned;	/* 1: derived is an allocation of its own */
@@ -60,22 +58,6 @@ struct anni_adam_priv {
 static size_t elem_bytes(int type)
 {
 	return type == ANNI_F32 ? 4 : type == ANNI_BF16 ? 2 : 1;
-}
-
-/* Size of one region of device memory (see the layout note in anni_adam_create); ANNI_REGION_GIB overrides. */
-static size_t region_bytes(void)
-{
-	static size_t r;
-
-	if (!r) {
-		const char *e = getenv("ANNI_REGION_GIB");
-		long g = e ? atol(e) : 16;
-
-		if (g < 1 || g > 64)
-			g = 16;
-		r = (size_t)g << 30;
-	}
-	return r;
 }
 
 static size_t round_up(size_t x, size_t a)
@@ -95,110 +77,112 @@ struct Sizes {
 	size_t	g_bytes;	/* one gradient slot, rounded up to 2 MiB */
 };
 
-/* One device allocation with the flats laid out in it. */
+/* One or two device allocations with the flats laid out in them. */
 struct Placement {
-	void	*arena;
-	size_t	total;
-	size_t	off_p, off_m, off_v, off_twin, off_g, off_gscale, off_segs, off_tiles, off_part,
-		off_state;
-	int	spread;
-	size_t	hole_off, hole_bytes;	/* spread: the rest of the tables' region, reserved and unused */
-	double	gbps;		/* what the probe measured (0: not probed) */
+	char	*a;		/* p, m, tables (split) or everything (compact) */
+	char	*b;		/* split: v, twins, gradient slots; NULL when compact */
+	size_t	a_bytes, b_bytes;
+	/* offsets from a: */
+	size_t	off_p, off_m, off_gscale, off_segs, off_tiles, off_part, off_state;
+	/* offsets from b (from a when compact): */
+	size_t	off_v, off_twin, off_g;
+	int	split;
+	double	ratio;		/* split: what alloc_apart_from measured */
+	double	gbps;		/* what the full-size probe measured (0: not probed) */
 };
 
 /*
-** Layout.  On MI355X a kernel that streams several arrays at once runs about 20 % faster
-** when the arrays lie in different 16 GiB regions of device memory than when two of them
-** share one (measured: 6.2 against 5.1 TB/s for this update; a kernel with a single
-** stream does not care), and another 4 % faster when no more than three of them lie in
-** the same group of four regions.  SPREAD therefore uses ONE allocation of a whole number
-** of regions: p, m, v in regions 0, 1, 2, the twins in region 4, the gradient slots from
-** region 5 on (region 3 holds only the small tables), so same-index elements of any two
-** flats are a whole number of regions apart.  The holes are reserved with it.  COMPACT
-** packs the flats at 2 MiB boundaries.
+** Layout.  MI355X's device memory behaves as three sections of 96 GiB, and a kernel that
+** streams several arrays at once runs about 15 % faster when its arrays are split over two
+** sections than when one section holds them all (placement.h).  SPLIT therefore uses TWO
+** allocations of exactly the size of their contents: p, m and the small tables in one, v, the
+** twins and the gradient slots in the other (16 + 18 of the update's 34 bytes per parameter),
+** the second one searched for in another section by timing the update on the zero-filled flats
+** themselves (alloc_apart_from).  Nothing is reserved beyond what the arena holds.  COMPACT is
+** one allocation with the flats at 2 MiB boundaries.
 */
-/*
-** Size of a spread arena.  The driver hands out device memory in naturally aligned
-** power-of-two blocks.  Up to six regions the arena is a 4-region block plus a 2-region
-** block (the layout keeps three flats in each); beyond that it is rounded up to one
-** power-of-two block, because a third, stray block was measured to make the gradient
-** slots that land in it 10 % slower than the others.
-*/
-static size_t spread_total(size_t need)
+static size_t tables_bytes(const Sizes &z)
 {
-	size_t p2 = region_bytes();
-
-	need = round_up(need, region_bytes());
-	if (need <= 6 * region_bytes())
-		return need;
-	while (p2 < need)
-		p2 <<= 1;
-	return p2;
-}
-
-static bool place(const Sizes &z, bool spread, Placement *pl)
-{
-	const size_t big = (size_t)2 << 20;
-	const size_t stride = spread ? round_up(z.p_bytes, region_bytes()) : 0;
-	const size_t tables = round_up((size_t)z.n_tensors * sizeof(float), 256)
+	return round_up((size_t)z.n_tensors * sizeof(float), 256)
 	    + round_up((size_t)z.n_tensors * sizeof(Seg), 256)
 	    + round_up((size_t)z.n_tiles * sizeof(int32_t), 256)
 	    + round_up((size_t)kMaxPartials * sizeof(double), 256) + kStateBytes;
+}
+
+static bool place(const Sizes &z, bool split, Placement *pl)
+{
+	const size_t big = (size_t)2 << 20;
+	void *mem = nullptr;
 
 	memset(pl, 0, sizeof(*pl));
-	if (spread) {
-		pl->off_p = 0;
-		pl->off_m = stride;
-		pl->off_v = 2 * stride;
-		pl->off_gscale = 3 * stride;		/* tables */
-		pl->off_twin = 4 * stride;
-		pl->off_g = (z.tw_bytes ? 5 : 4) * stride;
-		pl->total = spread_total(pl->off_g + (size_t)z.n_slots * z.g_bytes + big);
-		if (tables > stride)
-			return false;
+	pl->ratio = 1.0;
+	pl->off_p = 0;
+	pl->off_m = round_up(pl->off_p + z.p_bytes, big);
+	if (split) {
+		pl->off_gscale = round_up(pl->off_m + z.mv_bytes, big);
+		pl->off_v = 0;
 	} else {
-		pl->off_p = 0;
-		pl->off_m = round_up(pl->off_p + z.p_bytes, big);
 		pl->off_v = round_up(pl->off_m + z.mv_bytes, big);
-		pl->off_twin = round_up(pl->off_v + z.mv_bytes, big);
-		pl->off_g = round_up(pl->off_twin + z.tw_bytes, big);
-		pl->off_gscale = round_up(pl->off_g + (size_t)z.n_slots * z.g_bytes, big);
-		pl->total = pl->off_gscale + tables;
 	}
+	pl->off_twin = round_up(pl->off_v + z.mv_bytes, big);
+	pl->off_g = round_up(pl->off_twin + z.tw_bytes, big);
+	if (split)
+		pl->b_bytes = pl->off_g + (size_t)z.n_slots * z.g_bytes + big;
+	else
+		pl->off_gscale = round_up(pl->off_g + (size_t)z.n_slots * z.g_bytes, big);
 	pl->off_segs = pl->off_gscale + round_up((size_t)z.n_tensors * sizeof(float), 256);
 	pl->off_tiles = pl->off_segs + round_up((size_t)z.n_tensors * sizeof(Seg), 256);
 	pl->off_part = pl->off_tiles + round_up((size_t)z.n_tiles * sizeof(int32_t), 256);
 	pl->off_state = pl->off_part + round_up((size_t)kMaxPartials * sizeof(double), 256);
-	pl->spread = spread ? 1 : 0;
-	if (spread) {
-		pl->hole_off = round_up(pl->off_state + kStateBytes, big);
-		pl->hole_bytes = 4 * stride > pl->hole_off ? 4 * stride - pl->hole_off : 0;
-	}
-	if (hipMalloc(&pl->arena, pl->total) != hipSuccess) {
+	pl->a_bytes = pl->off_gscale + tables_bytes(z);
+	pl->split = split ? 1 : 0;
+	if (hipMalloc(&mem, pl->a_bytes) != hipSuccess) {
 		(void)hipGetLastError();
-		pl->arena = nullptr;
 		return false;
 	}
+	pl->a = (char *)mem;
+	if (split) {
+		/* p and m are still scratch: the search times the update on them and on each candidate */
+		pl->b = (char *)alloc_apart_from(pl->a, pl->off_gscale, pl->b_bytes, &pl->ratio);
+		if (!pl->b) {
+			(void)hipFree(pl->a);
+			pl->a = nullptr;
+			return false;
+		}
+	}
 	return true;
+}
+
+static void unplace(Placement *pl)
+{
+	if (pl->a)
+		(void)hip_ok(hipFree(pl->a), "arena hipFree");
+	if (pl->b)
+		(void)hip_ok(hipFree(pl->b), "arena hipFree");
+	pl->a = nullptr;
+	pl->b = nullptr;
 }
 
 /* Points the handle at a placement. */
 static void adopt(anni_adam *opt, const Sizes &z, const Placement &pl)
 {
 	anni_adam_priv *pv = opt->priv;
-	char *base = (char *)pl.arena;
+	char *base = pl.a;
+	char *second = pl.b ? pl.b : pl.a;
 
-	pv->arena = pl.arena;
-	pv->arena_bytes = pl.total;
-	pv->spread = pl.spread;
-	pv->hole = pl.hole_bytes ? base + pl.hole_off : nullptr;
-	pv->hole_bytes = pl.hole_bytes;
+	pv->arena = pl.a;
+	pv->arena2 = pl.b;
+	pv->arena_bytes = pl.a_bytes + pl.b_bytes;
+	pv->resident_bytes = z.p_bytes + 2 * z.mv_bytes + z.tw_bytes
+	    + (size_t)z.n * elem_bytes(opt->cfg.grad_type) + tables_bytes(z);
+	pv->split = pl.split;
+	pv->apart_ratio = pl.ratio;
 	pv->probe_gbps = pl.gbps;
 	opt->d_param = (float *)(base + pl.off_p);
 	opt->d_m = base + pl.off_m;
-	opt->d_v = base + pl.off_v;
-	opt->d_param_bf16 = z.tw_bytes ? base + pl.off_twin : nullptr;
-	pv->grad_slots = z.n_slots ? base + pl.off_g : nullptr;
+	opt->d_v = second + pl.off_v;
+	opt->d_param_bf16 = z.tw_bytes ? second + pl.off_twin : nullptr;
+	pv->grad_slots = z.n_slots ? second + pl.off_g : nullptr;
 	pv->grad_slot_bytes = z.g_bytes;
 	pv->n_grad_slots = z.n_slots;
 	opt->d_grad = pv->grad_slots;
@@ -213,15 +197,16 @@ static void adopt(anni_adam *opt, const Sizes &z, const Placement &pl)
 static bool init_contents(anni_adam *opt, const Sizes &z, const Placement &pl,
 	const std::vector<Seg> &segs, const std::vector<int32_t> &tile_seg)
 {
-	char *base = (char *)pl.arena;
+	char *base = pl.a;
+	char *second = pl.b ? pl.b : pl.a;
 	hipStream_t st = compute_stream();
 	std::vector<float> ones((size_t)z.n_tensors, 1.0f);
 
 	return launch_fill_bytes(st, base + pl.off_p, 0, z.p_bytes) == 0
 	    && launch_fill_bytes(st, base + pl.off_m, 0, z.mv_bytes) == 0
-	    && launch_fill_bytes(st, base + pl.off_v, 0, z.mv_bytes) == 0
-	    && (!z.tw_bytes || launch_fill_bytes(st, base + pl.off_twin, 0, z.tw_bytes) == 0)
-	    && (!z.n_slots || launch_fill_bytes(st, base + pl.off_g, 0,
+	    && launch_fill_bytes(st, second + pl.off_v, 0, z.mv_bytes) == 0
+	    && (!z.tw_bytes || launch_fill_bytes(st, second + pl.off_twin, 0, z.tw_bytes) == 0)
+	    && (!z.n_slots || launch_fill_bytes(st, second + pl.off_g, 0,
 	    (size_t)z.n_slots * z.g_bytes) == 0)
 	    && launch_fill_bytes(st, base + pl.off_part, 0, pl.off_state + kStateBytes - pl.off_part) == 0
 	    && hip_ok(hipMemcpyAsync(opt->d_gscale, ones.data(), (size_t)z.n_tensors * sizeof(float),
@@ -302,12 +287,6 @@ static anni_adam *create_body(const anni_tensor *tensors, int n_tensors,
 	const anni_adam_config *cfg, anni_adam **made)
 {
 	const size_t big = (size_t)2 << 20;	/* each flat starts on a 2 MiB boundary */
-	/* Spread arenas auditioned at most (a second one while the first stays below these figures). */
-	const int kTries = 2;
-	/* (good placements measure 6450-6570 / 6400-6460 / 6430-6520 in the three cases; others come 2 - 5 % lower) */
-	const double kGoodGBps = 6400.0;		/* all-f32 storage */
-	const double kGoodGBpsBf16 = 6350.0;		/* bf16 moments */
-	const double kGoodGBpsNarrow = 6400.0;		/* f32 moments, bf16 or fp8 gradients */
 	anni_adam *opt;
 	anni_adam_priv *pv;
 	Sizes z;
@@ -315,16 +294,16 @@ static anni_adam *create_body(const anni_tensor *tensors, int n_tensors,
 	std::vector<int32_t> tile_seg;
 	Placement pl;
 	int64_t n = 0;
-	bool want_spread;
+	bool want_split;
 	bool ok = false;
 
 	if (!tensors || n_tensors <= 0 || !cfg || !device_ready())
 		return nullptr;
-	(void)release_idle_slab();	/* the arena's own reservation is sized by what is free */
+	(void)release_idle_pools();	/* the search for the arena's second half looks at what is free */
 	if (cfg->grad_type < ANNI_F32 || cfg->grad_type > ANNI_FP8_E4M3
 	    || (cfg->moment_type != ANNI_F32 && cfg->moment_type != ANNI_BF16)
 	    || cfg->grad_slots < 0 || cfg->grad_slots > 4096
-	    || cfg->layout < ANNI_LAYOUT_AUTO || cfg->layout > ANNI_LAYOUT_SPREAD)
+	    || cfg->layout < ANNI_LAYOUT_AUTO || cfg->layout > ANNI_LAYOUT_SPLIT)
 		return nullptr;
 	for (int i = 0; i < n_tensors; i++) {
 		if (tensors[i].n < 0)
@@ -397,66 +376,34 @@ static anni_adam *create_body(const anni_tensor *tensors, int n_tensors,
 	memset(pv->h_state, 0, sizeof(StepState));
 
 	/*
-	** AUTO spreads flats of 256 MiB and more (smaller ones are not bandwidth critical),
-	** and only while the spread arena takes less than half of what is free.
+	** AUTO splits arenas whose parameter flat has 256 MiB or more (smaller ones are not
+	** bandwidth critical, and their probe launches would be too short to tell placements apart).
 	*/
-	want_spread = cfg->layout == ANNI_LAYOUT_SPREAD;
-	if (cfg->layout == ANNI_LAYOUT_AUTO && z.p_bytes >= ((size_t)256 << 20)) {
-		size_t free_b = 0, total_b = 0;
-		const size_t need = spread_total(5 * round_up(z.p_bytes, region_bytes())
-		    + (size_t)z.n_slots * z.g_bytes + ((size_t)64 << 20));
-
-		if (hipMemGetInfo(&free_b, &total_b) == hipSuccess && need <= free_b / 2)
-			want_spread = true;
-		(void)hipGetLastError();
-	}
-	if (want_spread) {
-		/*
-		** What the driver backs an allocation with is its choice and shows in the
-		** throughput: the same request can come back 5 - 20 % slower as a whole (every
-		** placement inside it), above all right after other large allocations were freed.
-		** So the update is timed on the fresh arena, and while the result is below par a
-		** SECOND arena is requested with the first still held -- freeing first and asking
-		** again was measured to hand back the same or worse memory -- and the faster of the
-		** two is kept.  Needs gradient slots to run on.
-		*/
-		const bool audition = z.n_slots > 0 && z.p_bytes >= ((size_t)256 << 20);
-		const double good = cfg->moment_type != ANNI_F32 ? kGoodGBpsBf16
-		    : cfg->grad_type != ANNI_F32 ? kGoodGBpsNarrow : kGoodGBps;
-
-		if (place(z, true, &pl)) {
-			adopt(opt, z, pl);
-			if (!init_contents(opt, z, pl, segs, tile_seg)) {
-				(void)hipFree(pl.arena);
-				pv->arena = nullptr;
-			} else {
-				ok = true;
-				pl.gbps = audition ? probe(opt) : 0.0;
+	want_split = cfg->layout == ANNI_LAYOUT_SPLIT
+	    || (cfg->layout == ANNI_LAYOUT_AUTO && z.p_bytes >= kPlaceMin);
+	if (want_split && place(z, true, &pl)) {
+		adopt(opt, z, pl);
+		if (init_contents(opt, z, pl, segs, tile_seg)) {
+			ok = true;
+			/* the update's throughput on the whole arena, for the record */
+			if (z.n_slots > 0 && z.p_bytes >= kPlaceMin) {
+				pl.gbps = probe(opt);
 				pv->probe_gbps = pl.gbps;
 			}
-		}
-		for (int k = 1; ok && audition && k < kTries && pl.gbps < good; k++) {
-			Placement cand;
-
-			if (!place(z, true, &cand))
-				break;			/* no room for a second one: keep what we have */
-			adopt(opt, z, cand);
-			cand.gbps = init_contents(opt, z, cand, segs, tile_seg) ? probe(opt) : 0.0;
-			(void)hipStreamSynchronize(compute_stream());
-			if (cand.gbps > pl.gbps) {
-				(void)hip_ok(hipFree(pl.arena), "arena hipFree");
-				pl = cand;
-			} else {
-				(void)hip_ok(hipFree(cand.arena), "arena hipFree");
-				adopt(opt, z, pl);
-			}
-			pv->probe_gbps = pl.gbps;
+		} else {
+			unplace(&pl);
+			pv->arena = nullptr;
+			pv->arena2 = nullptr;
 		}
 	}
-	if (!ok && cfg->layout != ANNI_LAYOUT_SPREAD) {
+	if (!ok && cfg->layout != ANNI_LAYOUT_SPLIT) {
 		if (place(z, false, &pl)) {
 			adopt(opt, z, pl);
 			ok = init_contents(opt, z, pl, segs, tile_seg);
+			if (!ok) {
+				unplace(&pl);
+				pv->arena = nullptr;
+			}
 		}
 	}
 	if (!ok) {
@@ -496,6 +443,8 @@ void anni_adam_free(anni_adam **popt)
 			(void)hipStreamSynchronize(compute_stream());
 		if (opt->priv->arena)
 			(void)hip_ok(hipFree(opt->priv->arena), "arena hipFree");
+		if (opt->priv->arena2)
+			(void)hip_ok(hipFree(opt->priv->arena2), "arena hipFree");
 		if (opt->priv->derived && opt->priv->derived_owned)
 			(void)hip_ok(hipFree(opt->priv->derived), "derived hipFree");
 		if (opt->priv->gq_scratch)
@@ -530,9 +479,24 @@ void *anni_adam_grad_slot(const anni_adam *opt, int k)
 	return opt->priv->grad_slots + (size_t)k * opt->priv->grad_slot_bytes;
 }
 
-int anni_adam_is_spread(const anni_adam *opt)
+int anni_adam_is_split(const anni_adam *opt)
 {
-	return opt && opt->priv ? opt->priv->spread : 0;
+	return opt && opt->priv ? opt->priv->split : 0;
+}
+
+double anni_adam_apart_ratio(const anni_adam *opt)
+{
+	return opt && opt->priv ? opt->priv->apart_ratio : 0.0;
+}
+
+size_t anni_adam_arena_bytes(const anni_adam *opt)
+{
+	return opt && opt->priv ? opt->priv->arena_bytes : 0;
+}
+
+size_t anni_adam_resident_bytes(const anni_adam *opt)
+{
+	return opt && opt->priv ? opt->priv->resident_bytes : 0;
 }
 
 double anni_adam_probe_gbps(const anni_adam *opt)
@@ -626,10 +590,7 @@ static int enable_derived_body(anni_adam *opt, const anni_pack *packs, int n_pac
 	off_pack = round_up(off_tamax + (fp8 ? (size_t)((opt->n + kTile - 1) / kTile) * kWaves
 	    * sizeof(float) : 0), (size_t)2 << 20);
 	total = off_pack + round_up((size_t)pack_elems * 2, 256) + 256;
-	if (pv->hole && total <= pv->hole_bytes) {
-		pv->derived = pv->hole;
-		pv->derived_owned = 0;
-	} else if (hipMalloc(&pv->derived, total) != hipSuccess) {
+	if (hipMalloc(&pv->derived, total) != hipSuccess) {
 		(void)hipGetLastError();
 		pv->derived = nullptr;
 		return -1;

@@ -18,10 +18,11 @@ void		set_compute_stream(hipStream_t st);
 /* Remembers the first HIP error for gpu_debug_last_error; returns err == hipSuccess. */
 bool		hip_ok(hipError_t err, const char *what);
 /*
-** gpu_malloc keeps its region slab reserved after the last block in it was freed; this gives it
-** back to the driver (true when there was one).  Called before other large reservations.
+** gpu_malloc keeps the chunks of its two pools reserved after the last block in them was freed;
+** this gives the empty ones back to the driver (true when there was one).  Called before other
+** large reservations.
 */
-bool		release_idle_slab(void);
+bool		release_idle_pools(void);
 
 } /* namespace anni */
 #endif

@@ -10,9 +10,11 @@
 #include <stdlib.h>
 #include <string.h>
 #include <mutex>
+#include <vector>
 #include "adam_kernels.h"
 #include "anni_gpu.h"
 #include "backend_state.h"
+#include "placement.h"
 
 namespace anni {
 
@@ -22,6 +24,7 @@ static hipStream_t g_own_stream;
 static hipStream_t g_stream;
 static std::mutex g_mu;			/* guards everything below */
 static char g_err[256];
+static std::mutex g_pool_mu;		/* guards gpu_malloc's pools; never taken with g_mu held */
 
 static void init_once(void)
 {
@@ -381,7 +384,7 @@ const char *gpu_backend_name(void)
 	return "hip-gfx950";
 }
 
-static size_t slab_idle_bytes_locked(void);
+static size_t pools_idle_bytes_locked(void);
 
 int gpu_mem_info(size_t *free_bytes, size_t *total_bytes)
 {
@@ -391,9 +394,9 @@ int gpu_mem_info(size_t *free_bytes, size_t *total_bytes)
 	if (!device_ready() || !hip_ok(hipMemGetInfo(&f, &t), "hipMemGetInfo"))
 		return -1;
 	{
-		std::lock_guard<std::mutex> lk(g_mu);
+		std::lock_guard<std::mutex> lk(g_pool_mu);
 
-		f += slab_idle_bytes_locked();	/* reserved, but given back on demand */
+		f += pools_idle_bytes_locked();	/* reserved, but given back on demand */
 	}
 	if (free_bytes)
 		*free_bytes = f;
@@ -473,101 +476,188 @@ void gpu_op_prof_dump(void)
 /* ---- memory --------------------------------------------------------------- */
 
 /*
-** Large blocks are spread over device memory.  lang/lm_adam.c asks for its five flats one
-** gpu_malloc at a time (d_param, d_grad, d_param_bf16, later d_m, d_v: lm_adam.c:222-229,
-** 295-297); packed next to each other they would share 16 GiB regions of device memory,
-** which costs the update ~20 % of its bandwidth on MI355X.  So the first large request
-** reserves one slab of six regions (4-region block + 2-region block) and every request of
-** kSpreadMin bytes or more gets a region of its own, in the order 0, 5, 4, 1, 2, 3 -- which
-** puts the caller's p, g, twin, m, v where the arena of anni_adam_create puts them (three
-** flats per 64 GiB group).  Anything that does not fit (no free region, larger than a
-** region, slab not available) is a plain hipMalloc.  ANNI_MALLOC_SPREAD=0 switches it off.
-** A slab whose last region was returned stays reserved (reserving and releasing 96 GiB costs
-** the driver about a second, and a caller that frees and re-allocates its flats would pay it
-** every time) until memory is wanted elsewhere: an allocation that fails, or an arena being
-** created, releases it first; gpu_mem_info counts it as free.
+** Large blocks, placed.  lang/lm_adam.c asks for its five flats one gpu_malloc at a time
+** (d_param, d_grad, d_param_bf16, later d_m, d_v: lm_adam.c:222-229,295-297).  On MI355X a kernel
+** that streams all of them runs ~15 % slower when they all lie in one of the three 96 GiB
+** sections of device memory than when they are split over two (placement.h).  So blocks of
+** kPlaceMin bytes and more are dealt to TWO pools, each new block to the pool that holds fewer
+** live bytes (p, twin, v | g, m for the caller above: 18 + 16 of the update's 34 bytes per
+** parameter).  A pool grows by chunks of four times the request that opens them; a chunk that
+** opens the second pool (or a later chunk of either) is looked for in another section than the
+** other pool's memory by timing the update on free space of both (alloc_apart_from).  Inside a
+** chunk blocks are handed out first-fit at 2 MiB boundaries and merged again when freed.  An
+** emptied chunk stays reserved (a caller that frees all its flats and allocates them again --
+** lm_adam_free and a new optimizer, the optional m/v offload -- would otherwise repeat the
+** search every time) until memory is wanted elsewhere: an allocation that fails, or an arena
+** being created, gives them back first; gpu_mem_info counts them as free.
+** ANNI_MALLOC_PLACE=0 switches all of this off (every block a plain hipMalloc).
 */
-static const size_t kSpreadMin = (size_t)256 << 20;
-static const size_t kRegion = (size_t)16 << 30;
-static const int kSpreadRegions = 6;
-static const int kSpreadOrder[kSpreadRegions] = { 0, 5, 4, 1, 2, 3 };
-static char *g_slab;
-static bool g_slab_tried;
-static bool g_region_used[kSpreadRegions];
-static int g_regions_live;
+struct PoolBlock {
+	size_t	off;
+	size_t	bytes;
+	bool	used;
+};
+struct PoolChunk {
+	char			*base;
+	size_t			bytes;
+	int			pool;
+	size_t			live;		/* bytes handed out */
+	std::vector<PoolBlock>	blocks;		/* sorted by offset, covering the chunk */
+};
+static std::vector<PoolChunk> g_chunks;
+static size_t g_pool_live[2];
 
-static bool spread_on(void)
+static bool place_on(void)
 {
 	static int on = -1;
 
 	if (on < 0) {
-		const char *e = getenv("ANNI_MALLOC_SPREAD");
+		const char *e = getenv("ANNI_MALLOC_PLACE");
 
 		on = (e && e[0] == '0') ? 0 : 1;
 	}
 	return on == 1;
 }
 
-/* Called with g_mu held.  Returns a region of the slab or nullptr. */
-static void *spread_take(size_t nbytes)
+/* First fit inside one chunk.  g_pool_mu held. */
+static void *chunk_take(PoolChunk &c, size_t need)
 {
-	if (!spread_on() || nbytes < kSpreadMin || nbytes > kRegion)
-		return nullptr;
-	if (!g_slab && !g_slab_tried) {
-		size_t free_b = 0, total_b = 0;
-		void *p = nullptr;
+	for (size_t i = 0; i < c.blocks.size(); i++) {
+		if (c.blocks[i].used || c.blocks[i].bytes < need)
+			continue;
+		if (c.blocks[i].bytes > need) {
+			const PoolBlock rest = { c.blocks[i].off + need, c.blocks[i].bytes - need, false };
 
-		g_slab_tried = true;
-		if (hipMemGetInfo(&free_b, &total_b) == hipSuccess
-		    && (size_t)kSpreadRegions * kRegion <= free_b / 2
-		    && hipMalloc(&p, (size_t)kSpreadRegions * kRegion) == hipSuccess)
-			g_slab = (char *)p;
-		(void)hipGetLastError();
-	}
-	if (!g_slab)
-		return nullptr;
-	for (int k = 0; k < kSpreadRegions; k++) {
-		const int r = kSpreadOrder[k];
-
-		if (!g_region_used[r]) {
-			g_region_used[r] = true;
-			g_regions_live++;
-			return g_slab + (size_t)r * kRegion;
+			c.blocks[i].bytes = need;
+			c.blocks.insert(c.blocks.begin() + (long)i + 1, rest);
 		}
+		c.blocks[i].used = true;
+		c.live += need;
+		g_pool_live[c.pool] += need;
+		return c.base + c.blocks[i].off;
 	}
 	return nullptr;
 }
 
-/* Called with g_mu held.  True when p was a region of the slab (now released). */
-static bool spread_give(void *p)
+/* The largest free block of the chunks of `pool`: scratch for the placement probe.  g_pool_mu held. */
+static char *pool_scratch(int pool, size_t *bytes)
 {
-	if (!g_slab || (char *)p < g_slab || (char *)p >= g_slab + (size_t)kSpreadRegions * kRegion)
-		return false;
-	const size_t off = (size_t)((char *)p - g_slab);
+	char *best = nullptr;
 
-	if (off % kRegion != 0 || !g_region_used[off / kRegion])
-		return false;
-	g_region_used[off / kRegion] = false;
-	g_regions_live--;
-	return true;
+	*bytes = 0;
+	for (PoolChunk &c : g_chunks) {
+		if (c.pool != pool)
+			continue;
+		for (const PoolBlock &b : c.blocks)
+			if (!b.used && b.bytes > *bytes) {
+				*bytes = b.bytes;
+				best = c.base + b.off;
+			}
+	}
+	return best;
 }
 
-/* Called with g_mu held.  Size of a slab that is reserved but holds no block. */
-static size_t slab_idle_bytes_locked(void)
+/* g_pool_mu held.  A block of a pool, or nullptr (the caller then allocates the plain way). */
+static void *pool_take(size_t nbytes)
 {
-	return g_slab && g_regions_live == 0 ? (size_t)kSpreadRegions * kRegion : 0;
+	const size_t need = (nbytes + ((size_t)2 << 20) - 1) & ~(((size_t)2 << 20) - 1);
+	const int pool = g_pool_live[1] < g_pool_live[0] ? 1 : 0;
+	size_t fr = 0, tt = 0, scratch_bytes = 0;
+	size_t chunk_bytes = 4 * need;
+	char *scratch;
+	void *mem = nullptr;
+	PoolChunk c;
+
+	for (PoolChunk &have : g_chunks)
+		if (have.pool == pool) {
+			void *p = chunk_take(have, need);
+
+			if (p)
+				return p;
+		}
+	if (hipMemGetInfo(&fr, &tt) != hipSuccess) {
+		(void)hipGetLastError();
+		return nullptr;
+	}
+	if (chunk_bytes > fr / 8)
+		chunk_bytes = need;		/* memory is short: no more than what is asked for */
+	if (chunk_bytes > fr / 2)
+		return nullptr;
+	scratch = pool_scratch(1 - pool, &scratch_bytes);
+	if (scratch) {
+		mem = alloc_apart_from(scratch, scratch_bytes, chunk_bytes, nullptr);
+	} else if (hipMalloc(&mem, chunk_bytes) != hipSuccess) {
+		(void)hipGetLastError();
+		mem = nullptr;
+	}
+	if (!mem)
+		return nullptr;
+	c.base = (char *)mem;
+	c.bytes = chunk_bytes;
+	c.pool = pool;
+	c.live = 0;
+	c.blocks.push_back(PoolBlock{ 0, chunk_bytes, false });
+	g_chunks.push_back(c);
+	return chunk_take(g_chunks.back(), need);
 }
 
-/* Called with g_mu held.  Gives an unused slab back to the driver; true when it did. */
-static bool slab_release_idle_locked(void)
+/* g_pool_mu held.  True when p was a block of a pool (now free again). */
+static bool pool_give(void *p)
 {
-	if (!g_slab || g_regions_live != 0)
-		return false;
-	(void)hipStreamSynchronize(g_stream);
-	(void)hipFree(g_slab);
-	g_slab = nullptr;
-	g_slab_tried = false;
-	return true;
+	for (PoolChunk &c : g_chunks) {
+		if ((char *)p < c.base || (char *)p >= c.base + c.bytes)
+			continue;
+		const size_t off = (size_t)((char *)p - c.base);
+
+		for (size_t i = 0; i < c.blocks.size(); i++) {
+			if (c.blocks[i].off != off || !c.blocks[i].used)
+				continue;
+			c.blocks[i].used = false;
+			c.live -= c.blocks[i].bytes;
+			g_pool_live[c.pool] -= c.blocks[i].bytes;
+			if (i + 1 < c.blocks.size() && !c.blocks[i + 1].used) {
+				c.blocks[i].bytes += c.blocks[i + 1].bytes;
+				c.blocks.erase(c.blocks.begin() + (long)i + 1);
+			}
+			if (i > 0 && !c.blocks[i - 1].used) {
+				c.blocks[i - 1].bytes += c.blocks[i].bytes;
+				c.blocks.erase(c.blocks.begin() + (long)i);
+			}
+			return true;
+		}
+		return false;		/* inside a chunk, but not the start of a live block */
+	}
+	return false;
+}
+
+/* g_pool_mu held.  Bytes of chunks that are reserved but hold no block. */
+static size_t pools_idle_bytes_locked(void)
+{
+	size_t idle = 0;
+
+	for (const PoolChunk &c : g_chunks)
+		if (c.live == 0)
+			idle += c.bytes;
+	return idle;
+}
+
+/* g_pool_mu held.  Gives the empty chunks back to the driver; true when there was one. */
+static bool pools_release_idle_locked(void)
+{
+	bool any = false;
+
+	for (size_t i = 0; i < g_chunks.size();) {
+		if (g_chunks[i].live != 0) {
+			i++;
+			continue;
+		}
+		if (!any)
+			(void)hipStreamSynchronize(g_stream);
+		(void)hipFree(g_chunks[i].base);
+		g_chunks.erase(g_chunks.begin() + (long)i);
+		any = true;
+	}
+	return any;
 }
 
 void *gpu_malloc(size_t nbytes)
@@ -576,21 +666,26 @@ void *gpu_malloc(size_t nbytes)
 
 	if (nbytes == 0 || !device_ready())
 		return nullptr;
-	{
-		std::lock_guard<std::mutex> lk(g_mu);
+	if (nbytes >= kPlaceMin && place_on()) {
+		batch_flush();			/* the placement probe runs on the compute stream */
+		try {
+			std::lock_guard<std::mutex> lk(g_pool_mu);
 
-		p = spread_take(nbytes);
+			p = pool_take(nbytes);
+		} catch (...) {
+			p = nullptr;
+		}
+		if (p)
+			return p;
 	}
-	if (p)
-		return p;
 	if (hipMalloc(&p, nbytes) != hipSuccess) {
 		bool released;
 
 		(void)hipGetLastError();
 		{
-			std::lock_guard<std::mutex> lk(g_mu);
+			std::lock_guard<std::mutex> lk(g_pool_mu);
 
-			released = slab_release_idle_locked();
+			released = pools_release_idle_locked();
 		}
 		if (!released || !hip_ok(hipMalloc(&p, nbytes), "hipMalloc")) {
 			if (!released)
@@ -616,7 +711,11 @@ void gpu_free(void *p)
 			g_twin_fp32 = nullptr;
 			g_twin_n = 0;
 		}
-		if (spread_give(p))
+	}
+	{
+		std::lock_guard<std::mutex> lk(g_pool_mu);
+
+		if (pool_give(p))
 			return;
 	}
 	(void)hip_ok(hipFree(p), "hipFree");
@@ -841,11 +940,11 @@ int gpu_adam_step_dev_bf16(ann_real *d_param, void *d_param_bf16, ann_real *d_gr
 
 namespace anni {
 
-bool release_idle_slab(void)
+bool release_idle_pools(void)
 {
-	std::lock_guard<std::mutex> lk(g_mu);
+	std::lock_guard<std::mutex> lk(g_pool_mu);
 
-	return slab_release_idle_locked();
+	return pools_release_idle_locked();
 }
 
 } /* namespace anni */

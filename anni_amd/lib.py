@@ -11,7 +11,7 @@ SO_PATH = os.path.join(HERE, "libanni_gpu_hip.so")
 
 F32, BF16, FP8_E4M3 = 0, 1, 2
 T_DECAY, T_TWIN, T_FP8TWIN = 1, 2, 4
-LAYOUT_AUTO, LAYOUT_COMPACT, LAYOUT_SPREAD = 0, 1, 2
+LAYOUT_AUTO, LAYOUT_COMPACT, LAYOUT_SPLIT = 0, 1, 2
 GPU_PREC_FP32, GPU_PREC_BF16 = 0, 1
 
 
@@ -92,8 +92,11 @@ _PROTOS = {
     "anni_adam_free": (None, [C.POINTER(C.POINTER(Adam))]),
     "anni_adam_tensor_offset": (C.c_int64, [C.POINTER(Adam), C.c_int]),
     "anni_adam_grad_slot": (C.c_void_p, [C.POINTER(Adam), C.c_int]),
-    "anni_adam_is_spread": (C.c_int, [C.POINTER(Adam)]),
+    "anni_adam_is_split": (C.c_int, [C.POINTER(Adam)]),
+    "anni_adam_apart_ratio": (C.c_double, [C.POINTER(Adam)]),
     "anni_adam_probe_gbps": (C.c_double, [C.POINTER(Adam)]),
+    "anni_adam_arena_bytes": (C.c_size_t, [C.POINTER(Adam)]),
+    "anni_adam_resident_bytes": (C.c_size_t, [C.POINTER(Adam)]),
     "anni_adam_bind_grad": (C.c_int, [C.POINTER(Adam), C.c_void_p]),
     "anni_adam_seed_twins": (C.c_int, [C.POINTER(Adam)]),
     "anni_adam_zero_grad": (C.c_int, [C.POINTER(Adam)]),

@@ -133,8 +133,20 @@ class LmAdam:
         return self.L.anni_adam_grad_slot(self.h, k)
 
     @property
-    def spread(self):
-        return bool(self.L.anni_adam_is_spread(self.h))
+    def split(self):
+        return bool(self.L.anni_adam_is_split(self.h))
+
+    @property
+    def apart_ratio(self):
+        return self.L.anni_adam_apart_ratio(self.h)
+
+    @property
+    def arena_bytes(self):
+        return self.L.anni_adam_arena_bytes(self.h)
+
+    @property
+    def resident_bytes(self):
+        return self.L.anni_adam_resident_bytes(self.h)
 
     @property
     def probe_gbps(self):

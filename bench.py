@@ -38,9 +38,33 @@ WORKLOADS = {
 }
 ELEM = {0: 4, 1: 2, 2: 1}
 # HBM bytes per launch of the update kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled
-# by what the counter reads for a plain copy kernel of known size (summaries under profiles/).
-TRAFFIC_BYTES = {"555m": 18907053045, "185m": 5712778091, "555m-bf16": 12236824127,
-                 "1p4b-fp8": 39599067321}
+# by what the counter reads for a plain copy kernel of known size: profiles/traffic.json, written
+# together with the summaries under profiles/ (per workload: scaled bytes read and written, the
+# scale factors, and a digest of the kernel sources the profiled library was built from).
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+KERNEL_SOURCES = ["adam_kernels.hip", "adam_kernels.h", "adam_math.h"]
+
+
+def kernel_sources_digest():
+    import hashlib
+    h = hashlib.sha1()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "anni_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def profiled_traffic(workload):
+    """(bytes per launch, digest of the profiled kernel sources, do today's sources match)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            t = json.load(f)[workload]
+    except (OSError, KeyError, ValueError):
+        return None, None, None
+    return (int(t["fetch_bytes"] + t["write_bytes"]), t.get("kernel_sources_sha1"),
+            t.get("kernel_sources_sha1") == kernel_sources_digest())
+
+
 STORAGE = {"185m": "f32 p/g/m/v + bf16 twin", "555m": "f32 p/g/m/v + bf16 twin",
            "555m-bf16": "f32 p, bf16 g/m/v + bf16 twin",
            "1p4b-fp8": "f32 p/m/v, fp8-e4m3 g with per-tensor scale + bf16 twin",
@@ -84,73 +108,61 @@ def fill_grad_slots(L, opt, tensors, count, grad_type, seed, first_step=0):
     return ptrs, scales
 
 
-def sweep_leg(L, workload, spec, rounds=3, timed=6):
-    """One arena, one process, the values of one switch taking turns: per value the mean step,
-    sum-of-squares and update time (ms, HIP events) over rounds x timed steps.  Two processes
-    differ by the memory they were given by a per cent or two, more than most settings do; runs
-    inside one process repeat to about 0.1 %."""
-    from anni_amd import layout
+def short_leg(L, workload, layout, steps=6, warmup=2, slots=4):
+    """A second arena in the same process (after the first was freed): `steps` timed steps of
+    `workload` on an arena of the given layout, HIP events per kernel.  For the all-f32 workloads."""
+    from anni_amd import layout as lay
+    from anni_amd import lm_adam
     from anni_amd.lm_adam import LmAdam
-    name, _, vals = spec.partition("=")
-    vals = [v for v in vals.split(",") if v != ""]
-    if not name.startswith("ANNI_") or not vals:
-        sys.exit("bench.py: --sweep wants NAME=V1,V2,... with an ANNI_* switch")
-    size, gt, mt, _nb, _ub = WORKLOADS[workload]
-    tensors = layout.tensors(size, "baseline")
-    slots = 8
-    opt = LmAdam(tensors, grad_type=gt, moment_type=mt, twins=True, skip_nonfinite=True,
-                 grad_slots=slots, beta2=0.95, weight_decay=0.1, grad_clip=1.0)
+    size, gt, mt, norm_bpp, upd_bpp = WORKLOADS[workload]
+    assert gt == 0 and mt == 0
+    tensors = lay.tensors(size, "baseline")
+    opt = LmAdam(tensors, twins=True, skip_nonfinite=True, grad_slots=slots,
+                 layout={"auto": 0, "compact": 1, "split": 2}[layout],
+                 beta2=0.95, weight_decay=0.1, grad_clip=1.0)
     n = opt.n
     assert L.anni_fill_normal_f32(opt.o.d_param, n, 20260101, 1, 0.0, 0.02) == 0
     opt.seed_twins()
     unit = 1.0 / (math.sqrt(n) * 1e-3)
-    step = 0
-    scales = []
-
-    def run(count):
-        nonlocal step
-        tot = [0.0, 0.0, 0.0]
-        for i in range(count):
-            k = (step + i) % slots
-            if gt == 2:
-                opt.o.d_gscale = scales[k].ptr
+    tot = [0.0, 0.0, 0.0]
+    wall = 0.0
+    done = 0
+    while done < warmup + steps:
+        count = min(slots, warmup + steps - done)
+        ring, _sc = fill_grad_slots(L, opt, tensors, count, 0, 20260101, done)
+        ptrs = (C.c_void_p * count)(*ring)
+        lr = (C.c_double * count)(*[lm_adam.step_lr(3e-4, done + i, 100, 1000, "cosine") for i in range(count)])
+        gs = (C.c_double * count)(*[unit * (1.7 if (done + i) % 2 else 0.6) for i in range(count)])
+        timed = [i for i in range(count) if done + i >= warmup]
+        if len(timed) < count:                           # the warm-up part of this batch
+            k = count - len(timed)
+            ms = C.c_float(0)
+            assert L.anni_adam_time_steps(opt.h, k, ptrs, k, lr, gs, C.byref(ms), None, None) == 0
+        if timed:
+            k0, k = timed[0], len(timed)
             ms, sa, sb = C.c_float(0), C.c_float(0), C.c_float(0)
-            rc = L.anni_adam_time_steps(opt.h, 1, (C.c_void_p * 1)(ring[k]), 1,
-                                        C.byref(C.c_double(1e-4)),
-                                        C.byref(C.c_double(unit * (1.7 if (step + i) % 2 else 0.6))),
-                                        C.byref(ms), C.byref(sa), C.byref(sb))
-            assert rc == 0, L.gpu_debug_last_error()
+            sub = (C.c_void_p * k)(*ring[k0:])
+            L.gpu_device_sync()
+            t0 = time.perf_counter()
+            assert L.anni_adam_time_steps(opt.h, k, sub, k, (C.c_double * k)(*lr[k0:]),
+                                          (C.c_double * k)(*gs[k0:]), C.byref(ms), C.byref(sa),
+                                          C.byref(sb)) == 0, L.gpu_debug_last_error()
+            L.gpu_device_sync()
+            wall += (time.perf_counter() - t0) * 1e3
             tot = [tot[0] + ms.value, tot[1] + sa.value, tot[2] + sb.value]
-        step += count
-        return [t / count for t in tot]
-
-    old = os.environ.get(name)
-    res = {v: [] for v in vals}
-    try:
-        for _round in range(rounds):
-            for v in vals:
-                os.environ[name] = v
-                L.anni_gpu_reload_switches()
-                for sc in scales:
-                    if sc is not None:
-                        sc.free()
-                ring, scales = fill_grad_slots(L, opt, tensors, slots, gt, 20260101, step)
-                run(2)
-                res[v].append(run(timed))
-    finally:
-        if old is None:
-            os.environ.pop(name, None)
-        else:
-            os.environ[name] = old
-        L.anni_gpu_reload_switches()
-    out = {"workload": workload, "switch": name, "placement_probe_GBps": round(opt.probe_gbps, 1),
-           "rounds": rounds, "timed_steps_per_round": timed, "values": {}}
-    for v in vals:
-        r = res[v]
-        out["values"][v] = {"step_ms": round(sum(x[0] for x in r) / len(r), 4),
-                            "sumsq_ms": round(sum(x[1] for x in r) / len(r), 4),
-                            "update_ms": round(sum(x[2] for x in r) / len(r), 4),
-                            "update_ms_rounds": [round(x[2], 4) for x in r]}
+        done += count
+    st = opt.sync_stats()
+    assert opt.t == warmup + steps and math.isfinite(st.last_grad_norm)
+    ms_step, upd_ms = wall / steps, tot[2] / steps
+    out = {"workload": workload, "params": n, "steps": steps, "warmup": warmup,
+           "layout": "split" if opt.split else "compact",
+           "placement_apart_ratio": round(opt.apart_ratio, 3),
+           "arena_bytes": opt.arena_bytes, "resident_bytes": opt.resident_bytes,
+           "ms_per_step": round(ms_step, 4),
+           "GBps": round(n * (norm_bpp + upd_bpp) / ms_step / 1e6, 1),
+           "frac": round(n * (norm_bpp + upd_bpp) / ms_step / 1e6 / HBM_PEAK_GBPS, 4),
+           "update_ms": round(upd_ms, 4), "sumsq_ms": round(tot[1] / steps, 4),
+           "update_frac": round(n * upd_bpp / upd_ms / 1e6 / HBM_PEAK_GBPS, 4)}
     opt.free()
     return out
 
@@ -369,7 +381,7 @@ def ckpt_leg(L, size="555m"):
 def ceilings(L, nbytes=8 << 30):
     """What this box delivers to the simplest kernels of the library: write-only (fill), copy
     (16-byte vectors, read + write) and read-only (the sum of squares), for comparison with the
-    update's mixed stream.  Every block sits in a 16 GiB region of its own."""
+    update's mixed stream."""
     a, b = L.gpu_malloc(nbytes), L.gpu_malloc(nbytes)
     assert a and b
     assert L.gpu_memset(a, 1, nbytes) == 0 and L.gpu_memset(b, 0, nbytes) == 0
@@ -419,9 +431,11 @@ def main():
                     help="timed steps (default 10 for the headline workload, 8 otherwise)")
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="555m", choices=sorted(WORKLOADS))
-    ap.add_argument("--layout", default="auto", choices=["auto", "compact", "spread"],
-                    help="arena layout (spread: every flat in its own 16 GiB region)")
+    ap.add_argument("--layout", default="auto", choices=["auto", "compact", "split"],
+                    help="arena layout (split: two allocations in different 96 GiB sections of device memory)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
+    ap.add_argument("--no-legs", action="store_true",
+                    help="skip the side legs of the headline workload (compact layout, 185m)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="only run the plain copy kernel over BYTES ten times (counter calibration)")
     ap.add_argument("--ckpt", action="store_true",
@@ -437,10 +451,6 @@ def main():
                     choices=["both", "fp8", "pack"],
                     help="the reference's own tensor list (separate Wq, Wk, Wv) with the fused "
                          "producers on: E4M3 twins of every matrix and a packed [Wq|Wk|Wv] per block")
-    ap.add_argument("--sweep", default=None, metavar="NAME=V1,V2,...",
-                    help="time the step under each value of one tuning switch (ANNI_TILES_PER_WG, "
-                         "ANNI_KEEP_MB, ANNI_REVERSE, ANNI_PIPE, ANNI_NT, ANNI_BLOCKS_PER_CU) on ONE "
-                         "arena in this process, the settings taking turns (one JSON line)")
     ap.add_argument("--ref-jsonl", default=None, metavar="FILE",
                     help="also append one row in the reference's bench-log schema (optimizer "
                          "phase only); steps are then timed one call each")
@@ -475,9 +485,6 @@ def main():
     if a.reference_caller_only:
         print(json.dumps(reference_caller_leg(L)))
         return
-    if a.sweep:
-        print(json.dumps({"sweep": sweep_leg(L, a.workload, a.sweep)}))
-        return
 
     size, gt, mt, norm_bpp, upd_bpp = WORKLOADS[a.workload]
     tensors = layout.tensors(size, "reference" if a.derived else "baseline")
@@ -496,14 +503,14 @@ def main():
                 packs.append((names.index("blk%d.%s" % (b, w)), d, pack_elems + k * d, 3 * d))
             pack_elems += 3 * d * d
     total = a.steps + a.warmup
-    # Gradient slots: one per step while they fit two 16 GiB regions of device memory (13 at 555M);
+    # Gradient slots: one per step while they fit 32 GiB of device memory (14 at 555M);
     # beyond that the steps run in batches, the slots being refilled between batches with the
     # clock stopped, so that any --steps keeps the arena, and with it the placement, the same.
     n_params = sum(t[1] for t in tensors)
     slot_bytes = -(-n_params * ELEM[gt] // (2 << 20)) * (2 << 20)
     n_slots = min(total, max(4, (32 << 30) // slot_bytes))
     opt = LmAdam(tensors, grad_type=gt, moment_type=mt, twins=True, skip_nonfinite=True,
-                 grad_slots=n_slots, layout={"auto": 0, "compact": 1, "spread": 2}[a.layout],
+                 grad_slots=n_slots, layout={"auto": 0, "compact": 1, "split": 2}[a.layout],
                  beta2=0.95, weight_decay=0.1, grad_clip=1.0)
     n = opt.n
     assert L.anni_fill_normal_f32(opt.o.d_param, n, 20260101, 1, 0.0, 0.02) == 0
@@ -592,6 +599,7 @@ def main():
     sumsq_ms = ms_sumsq / a.steps
     upd_bytes = n * upd_bpp + 2 * pack_elems
     upd_gbps = upd_bytes / (upd_ms * 1e-3) / 1e9
+    traffic, traffic_digest, traffic_current = profiled_traffic(a.workload)
     out = {
         "metric": "AdamW step HBM GB/s (algorithmic bytes / step time; AdamW + global-norm clip "
                   "+ decay + bf16 twins), %s param set" % a.workload,
@@ -602,9 +610,11 @@ def main():
         "config": {"workload": a.workload, "storage": STORAGE[a.workload], "params": n, "tensors": len(tensors),
                    "bytes_per_param": bpp, "clip": 1.0, "weight_decay": 0.1, "beta2": 0.95,
                    "lr": "3e-4 warmup100+cosine", "twins": "bf16 RNE on matrices",
-                   "layout": "spread" if opt.spread else "compact",
+                   "layout": "split" if opt.split else "compact",
+                   "placement_apart_ratio": round(opt.apart_ratio, 3),
                    "placement_probe_GBps": round(opt.probe_gbps, 1),
-                   "launches_per_step": 2},
+                   "arena_bytes": opt.arena_bytes, "resident_bytes": opt.resident_bytes,
+                   "grad_slots": n_slots, "launches_per_step": 2},
         "params_per_s": round(n / (ms_step * 1e-3), 1),
         "pct_of_hbm_peak": round(100.0 * step_gbps / HBM_PEAK_GBPS, 2),
         "event_ms_per_step": round(ev_ms / a.steps, 4),
@@ -613,7 +623,9 @@ def main():
                      "achieved": round(upd_gbps, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(upd_gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": None if a.derived else TRAFFIC_BYTES.get(a.workload),
+                     "traffic": None if a.derived else traffic,
+                     "profile_kernel_sources_sha1": None if a.derived else traffic_digest,
+                     "profile_matches_these_sources": None if a.derived else traffic_current,
                      "bytes_per_launch": upd_bytes, "avg_ms": round(upd_ms, 4)},
         "sumsq_kernel": {"avg_ms": round(sumsq_ms, 4), "bytes_per_launch": n * norm_bpp,
                          "achieved": round(n * norm_bpp / (sumsq_ms * 1e-3) / 1e9, 1)
@@ -648,6 +660,14 @@ def main():
         out["gpu_over_cpu"] = round(step_gbps / mt_out["value"], 1)
     opt.free()
     opt = None
+    if a.workload == "555m" and not a.derived and not a.no_legs:
+        # the same workload with every flat in ONE allocation, and the other parameter set the
+        # metric names, each on an arena of its own after the headline's was freed
+        try:
+            out["layout_compact"] = short_leg(L, "555m", "compact")
+            out["workloads"] = {"185m": short_leg(L, "185m", "auto")}
+        except Exception as e:                      # a side leg must never sink the bench line
+            out["side_legs_error"] = repr(e)
     if not a.no_cpu:
         try:
             ref_leg = reference_caller_leg(L)

@@ -38,18 +38,19 @@ extern "C" {
 #define ANNI_FP8_E4M3	2	/* OCP E4M3: bias 7, max 448, S.1111.111 = NaN, no infinities */
 
 /*
-** Arena layouts.  SPREAD puts every flat into its own 16 GiB region of device memory
-** (one allocation, holes included), which is what lets a kernel that streams all of
-** them at once reach full HBM speed on MI355X; COMPACT packs them.  AUTO spreads when
-** the parameter flat is at least 256 MiB and the spread arena takes less than half of
-** the free device memory.  What the driver backs the allocation with shows in the
-** throughput: creation times the update on the new arena and asks again (up to three
-** times, freeing in between) while it is slow; this needs gradient slots to run on.
-** Reserving and releasing ~100 GiB takes the driver a few seconds.
+** Arena layouts.  MI355X's device memory behaves as three sections of 96 GiB, and a kernel
+** that streams several arrays at once is ~15 % faster when they are split over two sections
+** than when one holds them all.  SPLIT makes two allocations of exactly the size of their
+** contents -- p, m and the tables in one; v, the twins and the gradient slots in the other -- and
+** looks for the second in another section by timing the update on the (still empty) flats:
+** candidates are requested with ballast in between until one is fast or memory runs low, and
+** everything but the arena is returned before anni_adam_create returns (for a moment up to
+** ~120 GiB more than the arena are held; with little memory free the search just ends sooner).
+** COMPACT is one allocation.  AUTO splits when the parameter flat has 256 MiB or more.
 */
 #define ANNI_LAYOUT_AUTO	0
 #define ANNI_LAYOUT_COMPACT	1
-#define ANNI_LAYOUT_SPREAD	2
+#define ANNI_LAYOUT_SPLIT	2
 
 /* Tensor flags. */
 #define ANNI_T_DECAY	1u	/* decoupled weight decay applies (the benchmark configurations: matrices only) */
@@ -101,7 +102,7 @@ typedef struct anni_adam {
 	int	last_skipped;
 	int	last_clipped;
 	anni_adam_config cfg;
-	/* the device arena: one allocation, each flat 2 MiB aligned (see ANNI_LAYOUT_*) */
+	/* the device arena: one or two allocations, each flat 2 MiB aligned (see ANNI_LAYOUT_*) */
 	float	*d_param;
 	void	*d_param_bf16;
 	void	*d_grad;
@@ -127,11 +128,21 @@ anni_adam	*anni_adam_create(const anni_tensor *tensors, int n_tensors,
 void	anni_adam_free(anni_adam **opt);
 /* Element offset of tensor i in every flat. */
 int64_t	anni_adam_tensor_offset(const anni_adam *opt, int i);
-/* Gradient slot k of the arena (k < cfg.grad_slots), else NULL; 1 when the layout came out SPREAD. */
+/* Gradient slot k of the arena (k < cfg.grad_slots), else NULL. */
 void	*anni_adam_grad_slot(const anni_adam *opt, int k);
-int	anni_adam_is_spread(const anni_adam *opt);
-/* GB/s of algorithmic traffic the update reached on this placement when the arena was created (0: not measured). */
+/* 1 when the layout came out SPLIT. */
+int	anni_adam_is_split(const anni_adam *opt);
+/*
+** What creation measured: time of the update with all flats in one block / time on this arena's
+** two blocks, on a probe of 64 M elements (>= 1.07: the halves lie in different sections; ~1.0:
+** no such memory was found; 1.0 exactly: compact or not measured), and the GB/s of algorithmic
+** traffic the update then reached on the whole arena (0: not measured; needs a gradient slot).
+*/
+double	anni_adam_apart_ratio(const anni_adam *opt);
 double	anni_adam_probe_gbps(const anni_adam *opt);
+/* Device memory the arena holds, and what one step touches (p, m, v, twins, one gradient flat, tables). */
+size_t	anni_adam_arena_bytes(const anni_adam *opt);
+size_t	anni_adam_resident_bytes(const anni_adam *opt);
 /* Use another gradient flat: a slot of the arena or an external one (n elements of grad_type); NULL = slot 0. */
 int	anni_adam_bind_grad(anni_adam *opt, void *d_grad);
 /*

@@ -89,19 +89,24 @@ def run_fp32_case(gpu, oracle, tensors, steps, clip, wd, gmul, grad_scale=1.0, s
     return n_clipped
 
 
-def test_spread_layout_gives_the_same_results(gpu, oracle):
-    """Every flat in its own 16 GiB region of device memory (one 96 GiB allocation)."""
+def test_split_layout_gives_the_same_results(gpu, oracle):
+    """Two allocations (p, m, tables | v, twins, gradient slots) instead of one."""
     from anni_amd import lib
-    opt = make(gpu, RAGGED, layout=lib.LAYOUT_SPREAD, grad_slots=2)
-    assert opt.spread and opt.grad_slot(1) - opt.grad_slot(0) >= 4 * opt.n
-    assert opt.o.d_m - opt.o.d_param == 16 << 30 and opt.o.d_v - opt.o.d_m == 16 << 30
-    assert opt.o.d_param_bf16 - opt.o.d_param == 64 << 30 and opt.grad_slot(0) - opt.o.d_param == 80 << 30
+    opt = make(gpu, RAGGED, layout=lib.LAYOUT_SPLIT, grad_slots=2)
+    n = opt.n
+    assert opt.split and opt.grad_slot(1) - opt.grad_slot(0) >= 4 * n
+    assert opt.o.d_m - opt.o.d_param >= 4 * n                     # first block: p, m
+    assert opt.o.d_param_bf16 - opt.o.d_v >= 4 * n                # second block: v, twins, slots
+    assert opt.grad_slot(0) - opt.o.d_param_bf16 >= 2 * n
+    assert not (opt.o.d_param <= opt.o.d_v < opt.o.d_param + 8 * n)
+    assert opt.arena_bytes >= opt.resident_bytes + 4 * n          # the second slot
+    assert opt.arena_bytes <= opt.resident_bytes + 4 * n + (16 << 20)   # nothing reserved beyond the contents
+    assert opt.apart_ratio == 1.0                                 # too small to be placed by measurement
     assert opt.grad_slot(2) is None
     opt.free()
-    n = sum(t[0] for t in RAGGED)
     base = 1.0 / (np.sqrt(n) * 1e-3)
     assert run_fp32_case(gpu, oracle, RAGGED, 4, clip=1.0, wd=0.1, gmul=[0.5 * base, 2.0 * base],
-                         layout=lib.LAYOUT_SPREAD) == 2
+                         layout=lib.LAYOUT_SPLIT) == 2
 
 
 def test_config1_no_clip_ragged(gpu, oracle):

@@ -377,40 +377,56 @@ def test_the_unchanged_reference_caller_on_this_backend(gpu, oracle):
     gpu.gpu_adam_set_weight_decay(0.0)
 
 
-def test_large_allocations_are_spread_over_regions(gpu):
-    """gpu_malloc gives every large block a 16 GiB region of its own, in the order that puts the
-    caller's p, g, twin, m, v (lm_adam.c:222-229,295-297) three to a 64 GiB group."""
+def test_large_allocations_are_dealt_to_two_pools(gpu):
+    """gpu_malloc deals blocks of 256 MiB and more to two pools of chunks, each block to the pool
+    with fewer live bytes: the caller's p, g, twin, m, v (lm_adam.c:222-229,295-297) end up as
+    p, twin, v | g, m, and the second pool's chunk is looked for in another section of device
+    memory.  Freed blocks are reused, empty chunks stay reserved and count as free."""
+    from anni_amd.lm_adam import LmAdam
+    opt = LmAdam([(4096, 3)])                            # creating an arena returns idle chunks first
+    opt.free()
+    fr0, tt = C.c_size_t(0), C.c_size_t(0)
+    assert gpu.gpu_mem_info(C.byref(fr0), C.byref(tt)) == 0
     n = 160 * 1000 * 1000                                # every block >= 256 MiB
     sizes = [4 * n, 4 * n, 2 * n, 4 * n, 4 * n]
     ptrs = [gpu.gpu_malloc(sz) for sz in sizes]
     assert all(ptrs)
-    base = ptrs[0]
-    assert [(p - base) >> 34 for p in ptrs] == [0, 5, 4, 1, 2]
-    assert all((p - base) % (1 << 34) == 0 for p in ptrs)
+    chunk = 4 * (-(-4 * n // (2 << 20)) * (2 << 20))     # four times the request that opened it
+    a, b = ptrs[0], ptrs[1]                              # first block of each pool = start of its chunk
+
+    def pool_of(p):
+        return 0 if a <= p < a + chunk else 1 if b <= p < b + chunk else None
+    assert [pool_of(p) for p in ptrs] == [0, 1, 0, 1, 0]
+    assert not (a <= b < a + chunk) and not (b <= a < b + chunk)
+    assert all(p % (2 << 20) == 0 for p in ptrs)
     small = gpu.gpu_malloc(1 << 20)                      # small blocks are ordinary allocations
-    assert small and not (base <= small < base + (6 << 34))
+    assert small and pool_of(small) is None
     gpu.gpu_free(ptrs[1])
-    again = gpu.gpu_malloc(4 * n)                        # a freed region is reused
+    again = gpu.gpu_malloc(4 * n)                        # a freed block is reused (first fit)
     assert again == ptrs[1]
     # the memory is usable: fill and read back the ends of one block
     assert gpu.gpu_memset(ptrs[3], 0x5a, 4 * n) == 0
     tail = np.zeros(16, np.uint8)
     assert gpu.gpu_memcpy_d2h(tail.ctypes.data, ptrs[3] + 4 * n - 16, 16) == 0 and (tail == 0x5a).all()
-    fr_live, fr_idle, tt = C.c_size_t(0), C.c_size_t(0), C.c_size_t(0)
+    head = np.zeros(16, np.uint8)
+    assert gpu.gpu_memset(ptrs[4], 0x33, 4 * n) == 0     # the neighbour in the other pool's chunk is untouched
+    assert gpu.gpu_memcpy_d2h(head.ctypes.data, ptrs[3], 16) == 0 and (head == 0x5a).all()
+    fr_live = C.c_size_t(0)
     assert gpu.gpu_mem_info(C.byref(fr_live), C.byref(tt)) == 0
+    assert fr0.value - fr_live.value <= 2 * chunk + (64 << 20)     # two chunks, nothing else
     for p in [ptrs[0], again, ptrs[2], ptrs[3], ptrs[4], small]:
         gpu.gpu_free(p)
-    # everything returned: the slab stays reserved for the next large request (no driver round
-    # trip), is reported as free memory, and goes back to the driver when an arena is created
+    # everything returned: the chunks stay reserved for the next large request, are reported as
+    # free memory, and go back to the driver when an arena is created
+    fr_idle = C.c_size_t(0)
     assert gpu.gpu_mem_info(C.byref(fr_idle), C.byref(tt)) == 0
-    assert fr_idle.value >= fr_live.value + (6 << 34)
+    assert fr_idle.value >= fr_live.value + 2 * chunk - (64 << 20)
     fresh = gpu.gpu_malloc(4 * n)
-    assert fresh == base
+    assert fresh == a                                    # merged back into one free block
     gpu.gpu_free(fresh)
-    from anni_amd.lm_adam import LmAdam
     opt = LmAdam([(4096, 3)])
     opt.free()
-    again2 = gpu.gpu_malloc(4 * n)                       # a new slab after the release
+    again2 = gpu.gpu_malloc(4 * n)                       # new chunks after the release
     assert again2
     gpu.gpu_free(again2)
 
@@ -462,10 +478,10 @@ def test_small_copies_are_batched_in_order(gpu):
 def test_malloc_and_free_from_many_threads(gpu):
     """gpu_malloc / gpu_free are called from OpenMP threads in the reference (gpu_cuda.cu:2644-2645):
     eight threads allocate, fill, check and free blocks of mixed sizes, the large ones out of the
-    region slab; afterwards the device holds what it held before."""
+    two pools; afterwards the device holds what it held before."""
     import threading
     fr0, tt = C.c_size_t(0), C.c_size_t(0)
-    hold = gpu.gpu_malloc(300 << 20)                 # keeps the region slab alive while the threads churn
+    hold = gpu.gpu_malloc(300 << 20)                 # keeps one chunk alive while the threads churn
     assert hold
     gpu.gpu_device_sync()
     assert gpu.gpu_mem_info(C.byref(fr0), C.byref(tt)) == 0

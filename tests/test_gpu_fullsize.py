@@ -89,7 +89,10 @@ def test_config3_555m_step_and_properties(gpu, oracle):
     parameters, then size-independent properties of a skipped and a clipped step."""
     opt, tensors, segs, mask = setup(gpu, "555m", skip_nonfinite=True)
     n = opt.n
-    assert opt.spread                                  # large arenas take the spread layout
+    # large arenas are split over two sections of device memory, found by measurement, and hold
+    # nothing beyond their contents
+    assert opt.split and opt.apart_ratio >= 1.05, opt.apart_ratio
+    assert opt.arena_bytes <= opt.resident_bytes + (16 << 20)
     P, M, V = opt.download("param"), np.zeros(n, np.float32), np.zeros(n, np.float32)
     O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True,
                       tensors=segs, threads=THREADS, simd=oracle.cpu_simd())
