@@ -11,6 +11,7 @@
 #include <stdlib.h>
 #include <string.h>
 #include <unistd.h>
+#include <mutex>
 #include <new>
 #include <vector>
 #include "adam_kernels.h"
@@ -280,6 +281,8 @@ static double probe(const anni_adam *opt)
 	return ms > 0.0f ? 2.0 * bytes / (ms * 1e-3) / 1e9 : 0.0;
 }
 
+static void *scratch_on_this_device(void);
+
 extern "C" {
 
 /* *made holds the handle as soon as it exists, so the caller can release it if this throws. */
@@ -374,6 +377,8 @@ static anni_adam *create_body(const anni_tensor *tensors, int n_tensors,
 		return nullptr;
 	}
 	memset(pv->h_state, 0, sizeof(StepState));
+	if (cfg->grad_type == ANNI_FP8_E4M3)
+		(void)scratch_on_this_device();	/* set-up of anni_adam_quantize_grads_static on this device */
 
 	/*
 	** AUTO splits arenas whose parameter flat has 256 MiB or more (smaller ones are not
@@ -647,21 +652,48 @@ int anni_adam_zero_grad(anni_adam *opt)
 	    (size_t)opt->n * elem_bytes(opt->cfg.grad_type));
 }
 
+/*
+** The passes that keep the E4M3 weight twins, pointed at the gradients and at every tensor:
+** maxima of whole tiles per wavefront (tiles shared by tensors raise the tensors' words
+** directly), folded into one word per tensor, then scale_t = max(amax_t / 448, 1e-12) and
+** q = E4M3(x * (1 / scale_t)) -- the arithmetic of anni_fp8_quantize on each tensor.  `work` holds
+** one word per tensor (cleared here, on the stream) and, 256-byte aligned behind them, the tile
+** maxima (every one that is read was written by this call).
+*/
+static int quantize_grads_into(anni_adam *opt, const float *d_src, void *work)
+{
+	anni_adam_priv *pv = opt->priv;
+	hipStream_t st = compute_stream();
+	const size_t amax_bytes = round_up((size_t)opt->n_tensors * sizeof(uint32_t), 256);
+	Flat f;
+
+	memset(&f, 0, sizeof(f));
+	f.p = const_cast<float *>(d_src);
+	f.n = opt->n;
+	f.segs = pv->d_segs;
+	f.tile_seg = pv->d_tile_seg;
+	f.der.wamax = (uint32_t *)work;
+	f.der.tile_amax = (float *)((char *)work + amax_bytes);
+	if (launch_fill_bytes(st, f.der.wamax, 0, (size_t)opt->n_tensors * sizeof(uint32_t)) != 0
+	    || launch_derive(st, f, 0u) != 0
+	    || launch_amax_fold(st, f, nullptr, 0u) != 0
+	    || launch_fp8_twins(st, f, (uint8_t *)opt->d_grad, opt->d_gscale, f.der.wamax,
+	    opt->n_tensors, nullptr, 0u) != 0)
+		return -1;
+	return 0;
+}
+
 int anni_adam_quantize_grads(anni_adam *opt, const float *d_src)
 {
 	anni_adam_priv *pv;
-	hipStream_t st;
-	Flat f;
-	size_t amax_bytes;
 
 	if (!opt || !opt->priv || !d_src || !opt->d_grad || !opt->d_gscale || !device_ready()
 	    || opt->cfg.grad_type != ANNI_FP8_E4M3 || ((uintptr_t)d_src & 15) != 0)
 		return -1;
 	pv = opt->priv;
-	st = compute_stream();
-	amax_bytes = round_up((size_t)opt->n_tensors * sizeof(uint32_t), 256);
 	if (!pv->gq_scratch) {
 		const size_t n_tiles = (size_t)((opt->n + kTile - 1) / kTile);
+		const size_t amax_bytes = round_up((size_t)opt->n_tensors * sizeof(uint32_t), 256);
 		void *d = nullptr;
 
 		if (!hip_ok(hipMalloc(&d, amax_bytes + n_tiles * kWaves * sizeof(float)),
@@ -671,26 +703,61 @@ int anni_adam_quantize_grads(anni_adam *opt, const float *d_src)
 		}
 		pv->gq_scratch = d;
 	}
-	/*
-	** The passes that keep the E4M3 weight twins, pointed at the gradients and at every tensor:
-	** maxima of whole tiles per wavefront (tiles shared by tensors raise the tensors' words
-	** directly), folded into one word per tensor, then scale_t = max(amax_t / 448, 1e-12) and
-	** q = E4M3(x * (1 / scale_t)) -- the arithmetic of anni_fp8_quantize on each tensor.
-	*/
-	memset(&f, 0, sizeof(f));
-	f.p = const_cast<float *>(d_src);
-	f.n = opt->n;
-	f.segs = pv->d_segs;
-	f.tile_seg = pv->d_tile_seg;
-	f.der.wamax = (uint32_t *)pv->gq_scratch;
-	f.der.tile_amax = (float *)((char *)pv->gq_scratch + amax_bytes);
-	if (launch_fill_bytes(st, f.der.wamax, 0, (size_t)opt->n_tensors * sizeof(uint32_t)) != 0
-	    || launch_derive(st, f, 0u) != 0
-	    || launch_amax_fold(st, f, nullptr, 0u) != 0
-	    || launch_fp8_twins(st, f, (uint8_t *)opt->d_grad, opt->d_gscale, f.der.wamax,
-	    opt->n_tensors, nullptr, 0u) != 0)
+	return quantize_grads_into(opt, d_src, pv->gq_scratch);
+}
+
+/*
+** The same without any allocation: the work area is a fixed array in device memory that every
+** GPU the library runs on holds from the moment the library is loaded until the process ends.
+*/
+static __device__ __align__(256) unsigned char scratch[ANNI_QUANT_STATIC_BYTES];
+
+static const int kScratchDevices = 64;
+static void *g_scratch_ptr[kScratchDevices];	/* the array's address on each device (the name itself is no device address) */
+static std::mutex g_scratch_mu;
+
+/* The address of `scratch` on the current device, looked up once per device; NULL on failure. */
+static void *scratch_on_this_device(void)
+{
+	int dev = -1;
+	void *ptr = nullptr;
+
+	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kScratchDevices) {
+		(void)hipGetLastError();
+		return nullptr;
+	}
+	std::lock_guard<std::mutex> lk(g_scratch_mu);
+
+	if (g_scratch_ptr[dev])
+		return g_scratch_ptr[dev];
+	if (!hip_ok(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) {
+		(void)hipGetLastError();
+		return nullptr;
+	}
+	g_scratch_ptr[dev] = ptr;
+	return ptr;
+}
+
+int anni_adam_quantize_grads_static(anni_adam *opt, const float *d_src)
+{
+	void *work;
+	size_t need;
+
+	if (!opt || !opt->priv || !d_src || !opt->d_grad || !opt->d_gscale || !device_ready()
+	    || opt->cfg.grad_type != ANNI_FP8_E4M3 || ((uintptr_t)d_src & 15) != 0)
 		return -1;
-	return 0;
+	need = round_up((size_t)opt->n_tensors * sizeof(uint32_t), 256)
+	    + (size_t)((opt->n + kTile - 1) / kTile) * kWaves * sizeof(float);
+	if (opt->n > ANNI_QUANT_STATIC_MAX_ELEMS || opt->n_tensors > ANNI_QUANT_STATIC_MAX_TENSORS
+	    || need > sizeof(scratch)) {
+		(void)hip_ok(hipErrorInvalidValue, "anni_adam_quantize_grads_static: more than "
+		    "ANNI_QUANT_STATIC_MAX_ELEMS elements or ANNI_QUANT_STATIC_MAX_TENSORS tensors");
+		return -1;
+	}
+	work = scratch_on_this_device();
+	if (!work)
+		return -1;
+	return quantize_grads_into(opt, d_src, work);
 }
 
 } /* extern "C" */

@@ -101,6 +101,7 @@ _PROTOS = {
     "anni_adam_seed_twins": (C.c_int, [C.POINTER(Adam)]),
     "anni_adam_zero_grad": (C.c_int, [C.POINTER(Adam)]),
     "anni_adam_quantize_grads": (C.c_int, [C.POINTER(Adam), C.c_void_p]),
+    "anni_adam_quantize_grads_static": (C.c_int, [C.POINTER(Adam), C.c_void_p]),
     "anni_adam_step_scaled": (C.c_int, [C.POINTER(Adam), C.c_double, C.c_double]),
     "anni_adam_step": (C.c_int, [C.POINTER(Adam), C.c_double]),
     "anni_adam_sync_stats": (C.c_int, [C.POINTER(Adam)]),

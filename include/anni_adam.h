@@ -176,6 +176,22 @@ int	anni_adam_zero_grad(anni_adam *opt);
 */
 int	anni_adam_quantize_grads(anni_adam *opt, const float *d_src);
 /*
+** anni_adam_quantize_grads for callers that cannot allocate device memory (a stream under HIP
+** graph capture, a tight serving loop, a harness that forbids hipMalloc): same arguments, same
+** codes and scales, but the work area (one word per tensor + 16 bytes per tile of 4096 elements)
+** is a fixed array of ANNI_QUANT_STATIC_BYTES in device memory that every GPU the library runs on
+** holds until the process ends, instead of a block allocated at the first call.  No counterpart
+** in the reference.  Calls no hipMalloc / hipFree; -1 (gpu_debug_last_error says why) for an
+** optimizer of more than ANNI_QUANT_STATIC_MAX_ELEMS elements or ANNI_QUANT_STATIC_MAX_TENSORS
+** tensors.  All calls on one GPU share the array: calls that overlap in time (two optimizers on
+** two streams) race; calls one after the other on the compute stream are fine, each clears what
+** it needs cleared.
+*/
+#define ANNI_QUANT_STATIC_MAX_ELEMS	((int64_t)1 << 31)
+#define ANNI_QUANT_STATIC_MAX_TENSORS	4096
+#define ANNI_QUANT_STATIC_BYTES		(16384 + (1 << 23))	/* the words + 2^31 / 4096 tiles x 16 bytes */
+int	anni_adam_quantize_grads_static(anni_adam *opt, const float *d_src);
+/*
 ** lm_adam_step_scaled (lm_adam.c:522-607): lr <= 0 returns 1 without advancing t;
 ** otherwise t++, [sum of squares when grad_clip > 0 or skip_nonfinite], update.
 ** Asynchronous on the compute stream: nothing is read back.
