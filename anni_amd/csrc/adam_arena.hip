@@ -216,7 +216,7 @@ static bool init_contents(anni_adam *opt, const Sizes &z, const Placement &pl,
 	    hipMemcpyHostToDevice, st), "segs")
 	    && hip_ok(hipMemcpyAsync(opt->priv->d_tile_seg, tile_seg.data(),
 	    (size_t)z.n_tiles * sizeof(int32_t), hipMemcpyHostToDevice, st), "tiles")
-	    && hip_ok(hipStreamSynchronize(st), "arena init");
+	    && hip_ok(sync_stream_and_deliver(), "arena init");
 }
 
 static void describe(const anni_adam *opt, Flat *f);
@@ -902,7 +902,7 @@ int anni_adam_sync_stats(anni_adam *opt)
 	st = compute_stream();
 	if (!hip_ok(hipMemcpyAsync(pv->h_state, pv->d_state, sizeof(StepState),
 	    hipMemcpyDeviceToHost, st), "stats d2h")
-	    || !hip_ok(hipStreamSynchronize(st), "stats sync"))
+	    || !hip_ok(sync_stream_and_deliver(), "stats sync"))
 		return -1;
 	opt->last_sumsq = pv->h_state->sumsq;
 	opt->last_grad_norm = pv->h_state->norm;
@@ -963,7 +963,7 @@ static int time_steps_body(anni_adam *opt, int count, void *const *grads, int n_
 	}
 	if (!per_kernel)
 		(void)hipEventRecord(ev[1], st);
-	if (!hip_ok(hipStreamSynchronize(st), "time_steps sync"))
+	if (!hip_ok(sync_stream_and_deliver(), "time_steps sync"))
 		rc = -1;
 	if (rc == 0) {
 		float ms = 0.0f;
@@ -1149,7 +1149,7 @@ static int import_pairs(anni_adam *opt, int64_t first, int64_t count, const Pair
 		    || !hip_ok(hipEventRecord(sg.ev[b], st), "import event")))
 			rc = -1;
 	}
-	if (!hip_ok(hipStreamSynchronize(st), "import sync"))
+	if (!hip_ok(sync_stream_and_deliver(), "import sync"))
 		rc = -1;
 	return rc;
 }
@@ -1304,6 +1304,12 @@ void anni_gpu_set_stream(void *hip_stream)
 {
 	if (device_ready())
 		set_compute_stream((hipStream_t)hip_stream);
+}
+
+void anni_gpu_flush(void)
+{
+	if (device_ready())
+		(void)compute_stream();		/* launches the pending batch of small copies, if any */
 }
 
 void anni_gpu_reload_switches(void)

@@ -12,6 +12,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
+#include <string.h>
 #include "adam_kernels.h"
 
 namespace anni {
@@ -289,6 +290,7 @@ struct SumsqArgs {
 	double		clip;
 	int		skip_nonfinite;
 	StepState	*state;
+	int		fence;		/* 1: the conservative hand-over (fences) instead of atomic accesses */
 };
 
 /*
@@ -304,7 +306,14 @@ struct SumsqArgs {
 ** which are performed where all dies see them: the partial is stored by an exchange whose result
 ** the ticket increment consumes (so the increment cannot be issued before the exchange has been
 ** performed), and the last workgroup reads the partials with atomic loads after its own increment
-** has returned.
+** has returned.  What this relies on, beyond the letter of the HIP memory model (which orders
+** relaxed atomics on different addresses only through fences): on gfx950 a returning atomic is
+** complete -- performed at the memory side that all dies share -- when its value arrives, an
+** instruction that consumes that value cannot issue earlier, and agent-scope atomic accesses are
+** performed there and not in a die's own level-two cache.  ANNI_FOLD=fence selects the hand-over
+** that needs none of this: plain stores of the partials, a release fence at device scope before
+** the tickets, an acquire fence in the last workgroup before it reads (+0.1 ms per launch at
+** 555M); the test of the switches holds the two against each other bit for bit.
 */
 constexpr int kFoldAhead = 8;	/* partials a lane of the last workgroup has in flight */
 
@@ -325,13 +334,19 @@ __device__ __forceinline__ void sumsq_finish(const SumsqArgs &a, double total, d
 			    : (unsigned int)kTicketGroups;
 			const unsigned int g = blockIdx.x % (unsigned int)kTicketGroups;
 			const unsigned int members = (gridDim.x - g + kTicketGroups - 1) / kTicketGroups;
-			const unsigned long long old = __hip_atomic_exchange(cells + blockIdx.x,
-			    (unsigned long long)__double_as_longlong(total), __ATOMIC_RELAXED,
-			    __HIP_MEMORY_SCOPE_AGENT);
 			unsigned int one = 1u;
 
-			/* ties the increment to the exchange's result: it waits for the exchange to return */
-			asm volatile("" : "+v"(one) : "v"(old));
+			if (a.fence) {
+				a.partials[blockIdx.x] = total;
+				__builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+			} else {
+				const unsigned long long old = __hip_atomic_exchange(cells + blockIdx.x,
+				    (unsigned long long)__double_as_longlong(total), __ATOMIC_RELAXED,
+				    __HIP_MEMORY_SCOPE_AGENT);
+
+				/* ties the increment to the exchange's result: it waits for the exchange to return */
+				asm volatile("" : "+v"(one) : "v"(old));
+			}
 			if (__hip_atomic_fetch_add(a.ticket + (1 + g) * kTicketStride, one, __ATOMIC_RELAXED,
 			    __HIP_MEMORY_SCOPE_AGENT) == members - 1u) {
 				/* the value just returned decided this branch: the next increment follows it */
@@ -345,6 +360,8 @@ __device__ __forceinline__ void sumsq_finish(const SumsqArgs &a, double total, d
 	__syncthreads();
 	if (!*last)
 		return;
+	if (a.fence)
+		__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 	/* lane l adds the partials l, l + 256, ... in that order, then the fixed tree over the lanes */
 	double acc = 0.0;
 
@@ -1201,6 +1218,7 @@ struct Switches {
 	int	keep_mb;	/* ANNI_KEEP_MB: how much of the gradients' tail the sum of squares leaves in the memory-side cache */
 	int	pipe;		/* ANNI_PIPE=0: narrow storage modes on the plain kernel; 2: the all-f32 mode pipelined too */
 	int	tiles_per_wg;	/* ANNI_TILES_PER_WG: tiles per workgroup of the update; 0 = the resident grid; -1 = the default */
+	int	fold_fence;	/* ANNI_FOLD=fence: the norm's second stage takes the partials over with fences (see sumsq_finish) */
 };
 static Switches g_sw;
 
@@ -1212,6 +1230,11 @@ void reload_switches(void)
 	g_sw.keep_mb = env_int("ANNI_KEEP_MB", 256, 0, 1 << 20);
 	g_sw.pipe = env_int("ANNI_PIPE", 1, 0, 2);
 	g_sw.tiles_per_wg = env_int("ANNI_TILES_PER_WG", -1, -1, 1 << 20);
+	{
+		const char *e = getenv("ANNI_FOLD");
+
+		g_sw.fold_fence = (e && strcmp(e, "fence") == 0) ? 1 : 0;
+	}
 	g_sw.loaded = 1;
 }
 
@@ -1325,6 +1348,7 @@ int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *parti
 	a.clip = 0.0;
 	a.skip_nonfinite = 0;
 	a.state = nullptr;
+	a.fence = sw().fold_fence;
 	if (fin) {
 		if (!fin->ticket || !fin->state || !aligned(fin->ticket, 128))
 			return -1;

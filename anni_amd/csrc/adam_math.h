@@ -43,14 +43,17 @@ struct Elem {
 ** a / b for a step constant b whose correctly rounded reciprocal rb the host supplies:
 ** q = a*rb, then one exact residual a - b*q folded back.  The result is a/b rounded to
 ** nearest unless a/b lies within ~2^-52 ulp of a rounding boundary (then it may be the
-** other neighbour): about one quotient in 2^52.  Used only where the update is bound by
-** arithmetic (narrow storage types); the all-f32 mode keeps the IEEE division.
+** other neighbour): about one quotient in 2^52.  A quotient that is not finite (a moment that
+** overflowed to infinity, a NaN) is returned as it is, as the division gives it -- its residual
+** would be inf - inf.  Used only where the update is bound by arithmetic (narrow storage
+** types); the all-f32 mode keeps the IEEE division.
 */
 __device__ __forceinline__ double div_by_const(double a, double b, double rb)
 {
 	const double q = a * rb;
+	const double r = __builtin_fma(__builtin_fma(-b, q, a), rb, q);
 
-	return __builtin_fma(__builtin_fma(-b, q, a), rb, q);
+	return __builtin_isfinite(q) ? r : q;
 }
 
 /*

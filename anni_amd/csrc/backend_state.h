@@ -13,6 +13,12 @@ namespace anni {
 /* True once a device is present and the compute stream exists. */
 bool		device_ready(void);
 hipStream_t	compute_stream(void);
+/*
+** Puts the pending batch of small copies on the stream, waits for the stream and hands the
+** batched device-to-host copies to their destinations: what every synchronisation inside the
+** library must do, so that a small gpu_memcpy_d2h_async is complete after ANY of them.
+*/
+hipError_t	sync_stream_and_deliver(void);
 /* NULL restores the library's own stream. */
 void		set_compute_stream(hipStream_t st);
 /* Remembers the first HIP error for gpu_debug_last_error; returns err == hipSuccess. */

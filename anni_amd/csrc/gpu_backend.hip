@@ -9,6 +9,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <atomic>
 #include <mutex>
 #include <vector>
 #include "adam_kernels.h"
@@ -53,7 +54,7 @@ bool device_ready(void)
 }
 
 static void batch_flush(void);
-static int g_batch_dir;
+static std::atomic<int> g_batch_dir;	/* written with g_mu held; read without it to see whether anything is pending */
 
 hipStream_t compute_stream(void)
 {
@@ -67,14 +68,22 @@ void set_compute_stream(hipStream_t st)
 	g_stream = st ? st : g_own_stream;
 }
 
+/* The same with g_mu already held (the mutex is not recursive). */
+static bool hip_ok_locked(hipError_t err, const char *what)
+{
+	if (err == hipSuccess)
+		return true;
+	if (!g_err[0])
+		snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(err));
+	return false;
+}
+
 bool hip_ok(hipError_t err, const char *what)
 {
 	if (err == hipSuccess)
 		return true;
 	std::lock_guard<std::mutex> lk(g_mu);
-	if (!g_err[0])
-		snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(err));
-	return false;
+	return hip_ok_locked(err, what);
 }
 
 /* ---- small copies, batched ------------------------------------------------- */
@@ -176,7 +185,7 @@ static void batch_flush_locked(void)
 	if (count > 0) {
 		hipLaunchKernelGGL(small_copy_kernel, dim3(count), dim3(256), 0, g_stream,
 		    g_desc + g_batch_first, g_stage, g_batch_dir == 1 ? 1 : 0);
-		(void)hip_ok(hipGetLastError(), "small copy batch");
+		(void)hip_ok_locked(hipGetLastError(), "small copy batch");
 	}
 	g_batch_first = g_desc_used;
 	g_batch_dir = 0;
@@ -244,7 +253,7 @@ static hipStream_t stream_for_op(void)
 }
 
 /* Waits for the stream and completes the batched D2H copies. */
-static hipError_t sync_stream_and_deliver(void)
+hipError_t sync_stream_and_deliver(void)
 {
 	hipError_t err;
 
@@ -853,6 +862,67 @@ unsigned gpu_param_epoch(void)
 {
 	std::lock_guard<std::mutex> lk(g_mu);
 	return g_epoch;
+}
+
+/* ANN_TWIN_CHECK=1: served twin slices are checked against a fresh conversion (gpu_cuda.cu:1946-1995). */
+static bool twin_check_on(void)
+{
+	static int on = -1;
+
+	if (on < 0) {
+		const char *e = getenv("ANN_TWIN_CHECK");
+
+		on = (e && e[0] == '1') ? 1 : 0;
+	}
+	return on == 1;
+}
+
+static void twin_check(const void *twin, const ann_real *fp32, size_t n)
+{
+	const size_t bytes = n * 2;
+	void *fresh = nullptr;
+	unsigned char *a, *b;
+	size_t bad = 0;
+
+	if (hipMalloc(&fresh, bytes) != hipSuccess) {
+		(void)hipGetLastError();
+		return;
+	}
+	a = (unsigned char *)malloc(bytes);
+	b = (unsigned char *)malloc(bytes);
+	if (a && b && launch_f32_to_bf16(stream_for_op(), (uint16_t *)fresh, fp32, (int64_t)n) == 0
+	    && hipMemcpyAsync(a, twin, bytes, hipMemcpyDeviceToHost, g_stream) == hipSuccess
+	    && hipMemcpyAsync(b, fresh, bytes, hipMemcpyDeviceToHost, g_stream) == hipSuccess
+	    && sync_stream_and_deliver() == hipSuccess) {
+		for (size_t i = 0; i < bytes; i++)
+			bad += a[i] != b[i];
+		if (bad)
+			fprintf(stderr, "[twin] STALE flat fp32=%p n=%zu bytes_diff=%zu\n",
+			    (const void *)fp32, n, bad);
+	}
+	(void)hipGetLastError();
+	free(a);
+	free(b);
+	(void)hipFree(fresh);
+}
+
+const void *anni_gpu_bf16_twin_of(const ann_real *fp32_dev, size_t n)
+{
+	const char *twin = nullptr;
+
+	if (!fp32_dev || n == 0 || !device_ready())
+		return nullptr;
+	{
+		std::lock_guard<std::mutex> lk(g_mu);
+
+		if (g_twin_bf16 && g_twin_fp32 && g_twin_n > 0 && fp32_dev >= g_twin_fp32
+		    && n <= (size_t)g_twin_n
+		    && (size_t)(fp32_dev - g_twin_fp32) <= (size_t)g_twin_n - n)
+			twin = (const char *)g_twin_bf16 + (size_t)(fp32_dev - g_twin_fp32) * 2u;
+	}
+	if (twin && twin_check_on())
+		twin_check(twin, fp32_dev, n);
+	return twin;
 }
 
 /* ---- the optimizer step -------------------------------------------------------- */

@@ -112,11 +112,13 @@ template <bool PROD> struct CsRows { static constexpr int n = 64; };
 
 /*
 ** Rows FIRST .. FIRST + COUNT - 1 of a chunk of the lane's column into registers, as raw buffer loads: the
-** descriptor (scalar registers) starts at the chunk's first row and ends with the matrix, the
-** row offset is a scalar, the lane supplies only its constant column offset -- no vector
-** arithmetic per load, and a row past the end reads as 0 without touching memory (those
-** registers are never added).  A select on a loaded value instead would make the wavefront
-** wait for the load on the spot.
+** descriptor (scalar registers) starts at the chunk's first row, the row offset is a scalar, the
+** lane supplies only its constant column offset -- no vector arithmetic per load.  A chunk that
+** runs past the matrix reads its last valid row again for the rows beyond it (those registers are
+** never added): the scalar row index is clamped, one scalar minimum per load, so every address
+** lies inside the matrix by construction.  (The descriptor's range check is not relied on for
+** this: it compares the vector offset only, the scalar offset takes no part in it.)  A select on
+** a loaded value instead would make the wavefront wait for the load on the spot.
 */
 template <bool PROD, int FIRST, int COUNT>
 __device__ __forceinline__ void colsum_fetch(float (&rx)[CsRows<PROD>::n], float (&ry)[CsRows<PROD>::n],
@@ -127,7 +129,9 @@ __device__ __forceinline__ void colsum_fetch(float (&rx)[CsRows<PROD>::n], float
 
 	if (r0 >= rows)
 		return;
-	const uint64_t left = (uint64_t)(rows - r0) * (uint64_t)cols * sizeof(float);
+	const int64_t rows_left = rows - r0;
+	const uint32_t last = (uint32_t)(rows_left < kCsRows ? rows_left - 1 : kCsRows - 1);
+	const uint64_t left = (uint64_t)rows_left * (uint64_t)cols * sizeof(float);
 	const uint32_t span = left < 0xffffffffull ? (uint32_t)left : 0xffffffffu;
 	const __amdgpu_buffer_rsrc_t bx = __builtin_amdgcn_make_buffer_rsrc(
 	    (void *)(x + r0 * cols), 0, (int)span, 0x00020000);
@@ -137,11 +141,13 @@ __device__ __forceinline__ void colsum_fetch(float (&rx)[CsRows<PROD>::n], float
 
 #pragma unroll
 	for (int i = FIRST; i < FIRST + COUNT; i++) {
+		const uint32_t row = (uint32_t)i < last ? (uint32_t)i : last;
+
 		rx[i] = __builtin_bit_cast(float,
-		    __builtin_amdgcn_raw_buffer_load_b32(bx, (int)col_bytes, (int)(i * pitch), 0));
+		    __builtin_amdgcn_raw_buffer_load_b32(bx, (int)col_bytes, (int)(row * pitch), 0));
 		if (PROD)
 			ry[i] = __builtin_bit_cast(float,
-			    __builtin_amdgcn_raw_buffer_load_b32(by, (int)col_bytes, (int)(i * pitch), 0));
+			    __builtin_amdgcn_raw_buffer_load_b32(by, (int)col_bytes, (int)(row * pitch), 0));
 	}
 }
 

@@ -82,6 +82,7 @@ _PROTOS = {
     "gpu_adam_seed_bf16_flat": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
     "gpu_half_wt_invalidate": (None, [C.c_void_p]),
     "gpu_param_epoch": (C.c_uint, []),
+    "anni_gpu_bf16_twin_of": (C.c_void_p, [C.c_void_p, C.c_size_t]),
     "gpu_adam_set_weight_decay": (None, [C.c_double]),
     "gpu_grad_sumsq": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_double)]),
     "gpu_adam_step_dev_bf16": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
@@ -123,6 +124,7 @@ _PROTOS = {
     "anni_lr_step": (C.c_double, [C.c_double, C.c_int]),
     "anni_gpu_stream": (C.c_void_p, []),
     "anni_gpu_set_stream": (None, [C.c_void_p]),
+    "anni_gpu_flush": (None, []),
     "anni_fill_normal_f32": (C.c_int, [C.c_void_p, C.c_int64, C.c_uint64, C.c_uint64,
                                        C.c_float, C.c_float]),
     "anni_copy_bytes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),

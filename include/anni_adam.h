@@ -230,6 +230,17 @@ double	anni_lr_step(double base_lr, int step);
 */
 void	*anni_gpu_stream(void);
 void	anni_gpu_set_stream(void *hip_stream);
+/*
+** gpu_memcpy_h2d / gpu_memcpy_d2h_async of 64 KiB or less are batched: they reach the stream
+** when the next entry point of this library enqueues something (lm_adam.c's per-vector copies
+** become two kernels per step that way).  Work that a caller puts on the stream handle ITSELF
+** (raw HIP calls, another library) does not pass through an entry point: call this first, it
+** puts the pending batch on the stream.  Batched device-to-host copies are complete after any
+** synchronising call of this library (gpu_stream_sync, gpu_device_sync, gpu_memcpy_d2h,
+** gpu_grad_sumsq, anni_adam_sync_stats, the checkpoint calls), not after a hipStreamSynchronize
+** of the caller's own.  ANNI_SMALL_COPY_BATCH=0 switches the batching off.
+*/
+void	anni_gpu_flush(void);
 
 /*
 ** Reads the kernels' tuning switches (ANNI_TILES_PER_WG, ANNI_KEEP_MB, ANNI_REVERSE, ANNI_PIPE,

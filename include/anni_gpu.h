@@ -90,6 +90,19 @@ int	gpu_adam_seed_bf16_flat(void *bf16, const ann_real *fp32, int n);
 void	gpu_half_wt_invalidate(const ann_real *fp32_dev);
 /* num/gpu.h:346 -- changes at every optimizer step. */
 unsigned	gpu_param_epoch(void);
+/*
+** The consumer side of the twin flat: the reference's GEMM wrappers ask half_wt_get for the
+** BF16 copy of a device FP32 operand (static in num/gpu_cuda.cu:2018-2034, so not part of
+** num/gpu.h; exported here for a GEMM backend written against this library).  A slice
+** [fp32_dev, fp32_dev + n) that lies inside the registered flat (gpu_adam_set_bf16_flat) is served
+** from the twin flat, bf16 + (fp32_dev - fp32_base) * 2 -- current after every step, no
+** conversion; any other pointer gets NULL once a flat is registered (it is an activation and
+** must not get a persistent twin), and NULL when none is.  gpu_free of either flat and
+** gpu_adam_set_bf16_flat(NULL, NULL, 0) end the service.  ANN_TWIN_CHECK=1 (gpu_cuda.cu:1946-1995):
+** every served slice is converted afresh on the device, compared, and a difference reported on
+** stderr as "[twin] STALE flat fp32=... n=... bytes_diff=..." (debug aid; synchronises).
+*/
+const void	*anni_gpu_bf16_twin_of(const ann_real *fp32_dev, size_t n);
 
 /* ---- the optimizer step ------------------------------------------------ */
 

@@ -402,6 +402,14 @@ class RefModelOnBackend:
     def last_grad_norm(self):
         return self.R.ref_model_last_norm(self.h)
 
+    def device_flats(self):
+        """(d_param, d_param_bf16) of the caller's optimizer, as integers."""
+        for name in ("ref_model_d_param", "ref_model_d_param_bf16"):
+            fn = getattr(self.R, name)
+            fn.argtypes = [C.c_void_p]
+            fn.restype = C.c_void_p
+        return self.R.ref_model_d_param(self.h), self.R.ref_model_d_param_bf16(self.h)
+
     def set_offload(self, on):
         """lm_adam_set_offload: a process-wide switch of the reference."""
         self.R.ref_set_offload(int(on))

@@ -184,6 +184,9 @@ int ref_model_n_segs(const ref_model *r) { return r->opt->n_segs; }
 int ref_model_t(const ref_model *r) { return r->opt->t; }
 int ref_model_on_device(const ref_model *r) { return r->opt->d_param != NULL; }
 double ref_model_last_norm(const ref_model *r) { return r->opt->last_grad_norm; }
+/* The caller's device flats (lang/lm_adam.h:43-44), for tests of what the backend serves from them. */
+void *ref_model_d_param(const ref_model *r) { return r->opt->d_param; }
+void *ref_model_d_param_bf16(const ref_model *r) { return r->opt->d_param_bf16; }
 
 /* seg i: off, n, 1 for a matrix / 0 for a vector. */
 void ref_model_seg(const ref_model *r, int i, long *off, long *n, int *is_mat)

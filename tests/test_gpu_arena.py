@@ -367,6 +367,50 @@ def test_multi_tensor_gradient_quantiser_equals_the_per_tensor_one(gpu, oracle):
     opt.free()
 
 
+@pytest.mark.parametrize("gt,mt", [(F32, BF16), (BF16, BF16), (FP8, F32)])
+def test_moment_overflow_follows_the_host_loop(gpu, oracle, gt, mt):
+    """A gradient so large that v overflows to infinity in float: the host loop then divides by
+    infinity and leaves p where it was (lm_adam.c:590-593), and so must the narrow storage modes,
+    whose division by the step constants is a reciprocal multiply with a residual (inf - inf)."""
+    n = 4096 * 3 + 5
+    rng = np.random.default_rng(5)
+    opt = make(gpu, [(n, 3)], grad_type=gt, moment_type=mt, beta2=0.95, weight_decay=0.1)
+    p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    opt.upload("param", p0)
+    g32 = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    big = rng.choice(n, 200, replace=False)
+    g32[big] = np.float32(1e20) * np.sign(g32[big])
+    segs = [(0, n, 1, 1.0)]
+    if gt == F32:
+        g_dev, g_or = g32, g32.copy()
+    elif gt == BF16:
+        g_dev = oracle.bf16_rne(g32)
+        g_or = g_dev.copy()
+    else:
+        g_dev, sc = oracle.fp8_quantize(g32)
+        g_or = g_dev.copy()
+        opt.upload("gscale", np.array([sc], np.float32))
+        segs = [(0, n, 1, float(sc))]
+    opt.upload("grad", g_dev)
+    P = p0.copy()
+    M = np.zeros(n, np.float32 if mt == F32 else np.uint16)
+    V = np.zeros(n, np.float32 if mt == F32 else np.uint16)
+    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_type=gt, moment_type=mt, tensors=segs)
+    for step in range(2):
+        if step:
+            opt.upload("grad", g_dev)
+            g_or = g_dev.copy()
+        opt.step_scaled(1e-3)
+        O.step(P, g_or, M, V, 1e-3)
+        got_v = opt.download("v")
+        vf = oracle.bf16_widen(got_v) if mt == BF16 else got_v
+        assert np.isinf(vf[big]).all()                           # the case is what it claims to be
+        assert same_bits(opt.download("param"), P), (gt, mt, step)
+        assert (opt.download("m").view(M.dtype) == M).all() and (got_v.view(V.dtype) == V).all()
+    assert np.isfinite(opt.download("param")).all()
+    opt.free()
+
+
 def test_fp8_decode_all_codes_on_device(gpu, oracle):
     """Every E4M3 byte through the kernel's decoder: with m = v = 0 and t = 1, m = (1-b1) * g."""
     opt = make(gpu, [(256, 0)], grad_type=FP8, beta1=0.5, beta2=0.5)

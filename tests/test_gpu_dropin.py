@@ -4,6 +4,7 @@ required tolerances (1e-6 relative on p/m/v, 1 bf16 ulp on twins, 1e-5 on the no
 summation order of the norm differs."""
 import ctypes as C
 import math
+import os
 
 import numpy as np
 import pytest
@@ -12,6 +13,7 @@ from helpers import GOLDEN_CASES, load_golden, same_bits, rel_err, bf16_ulp_diff
 
 pytestmark = pytest.mark.gpu
 
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 TOL_STATE = 1e-6     # required: FP32 master/m/v within 1e-6 relative per step
 TOL_NORM = 1e-5      # required: clip norm within 1e-5 relative
 
@@ -335,6 +337,55 @@ def test_seed_bf16_flat(gpu, oracle):
     assert gpu.gpu_adam_seed_bf16_flat(None, None, 5) == -1
 
 
+def test_twin_flat_is_served_and_checked(gpu, oracle, capfd):
+    """anni_gpu_bf16_twin_of: slices of the registered flat are served from the twin flat, anything
+    else and everything after gpu_free / a cleared registration gets NULL; with ANN_TWIN_CHECK=1
+    (read once per process: a child) a stale slice is reported as the reference reports it."""
+    import subprocess
+    import sys
+    n = 10000
+    x = (np.random.default_rng(9).standard_normal(n) * 0.02).astype(np.float32)
+    d, o = dev(gpu, x), dev(gpu, np.zeros(n, np.uint16))
+    assert gpu.anni_gpu_bf16_twin_of(d.ptr, n) is None               # nothing registered
+    gpu.gpu_adam_set_bf16_flat(o.ptr, d.ptr, n)
+    assert gpu.gpu_adam_seed_bf16_flat(o.ptr, d.ptr, n) == 0
+    assert gpu.anni_gpu_bf16_twin_of(d.ptr, n) == o.ptr
+    assert gpu.anni_gpu_bf16_twin_of(d.ptr + 4 * 100, 50) == o.ptr + 2 * 100
+    assert gpu.anni_gpu_bf16_twin_of(d.ptr + 4 * (n - 1), 1) == o.ptr + 2 * (n - 1)
+    assert gpu.anni_gpu_bf16_twin_of(d.ptr + 4 * (n - 1), 2) is None  # one element too far
+    assert gpu.anni_gpu_bf16_twin_of(d.ptr, 0) is None and gpu.anni_gpu_bf16_twin_of(None, 4) is None
+    assert gpu.anni_gpu_bf16_twin_of(o.ptr, 4) is None               # not an fp32 slice of the flat
+    gpu.gpu_adam_set_bf16_flat(None, None, 0)
+    assert gpu.anni_gpu_bf16_twin_of(d.ptr, n) is None
+    gpu.gpu_adam_set_bf16_flat(o.ptr, d.ptr, n)
+    o.free()                                                         # gpu_free forgets the registration
+    assert gpu.anni_gpu_bf16_twin_of(d.ptr, n) is None
+    d.free()
+    child = (
+        "import sys, numpy as np\n"
+        "sys.path.insert(0, %r)\n"
+        "from anni_amd import lib\n"
+        "from anni_amd.lm_adam import DeviceBuffer\n"
+        "L = lib.require_gpu()\n"
+        "n = 5000\n"
+        "x = np.linspace(-1, 1, n).astype(np.float32)\n"
+        "d, o = DeviceBuffer(4 * n), DeviceBuffer(2 * n)\n"
+        "d.upload(x)\n"
+        "L.gpu_adam_set_bf16_flat(o.ptr, d.ptr, n)\n"
+        "assert L.gpu_adam_seed_bf16_flat(o.ptr, d.ptr, n) == 0\n"
+        "assert L.anni_gpu_bf16_twin_of(d.ptr, n) == o.ptr\n"
+        "print('FRESH-DONE', flush=True)\n"
+        "d.upload((x * 3).astype(np.float32))\n"          # weights change behind the twins' back
+        "assert L.anni_gpu_bf16_twin_of(d.ptr + 400, 1000) == o.ptr + 200\n"
+        "L.gpu_adam_set_bf16_flat(None, None, 0)\n"
+    ) % ROOT
+    env = dict(os.environ, ANN_TWIN_CHECK="1")
+    r = subprocess.run([sys.executable, "-c", child], env=env, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr[-1500:]
+    stale = [ln for ln in r.stderr.splitlines() if ln.startswith("[twin] STALE flat")]
+    assert len(stale) == 1 and "n=1000" in stale[0], r.stderr[-1500:]
+
+
 def test_the_unchanged_reference_caller_on_this_backend(gpu, oracle):
     """lang/lm_adam.c itself, compiled from the reference tree and linked against
     libanni_gpu_hip.so instead of its CPU stub (oracle/_ref/libanni_ref_hip.so): its device path
@@ -473,6 +524,35 @@ def test_small_copies_are_batched_in_order(gpu):
     for off, ln, o in outs:
         assert (o == ref[off:off + ln]).all(), (off, ln)
     assert not d.download(np.uint8, 4096).any()
+
+
+def test_batched_copies_and_the_librarys_own_syncs(gpu):
+    """A small gpu_memcpy_d2h_async is complete after ANY synchronising call of the library, the
+    arena's included, and anni_gpu_flush puts a pending small upload on the stream for work the
+    caller enqueues on the stream handle itself."""
+    from anni_amd.lm_adam import DeviceBuffer, LmAdam
+    d = DeviceBuffer(4096)
+    src = np.arange(4096, dtype=np.uint8)
+    d.upload(src)
+    opt = LmAdam([(4096, 3)])
+    out = np.zeros(1000, np.uint8)
+    assert gpu.gpu_memcpy_d2h_async(out.ctypes.data, d.ptr + 96, 1000) == 0
+    opt.sync_stats()                                     # not one of the gpu_* syncs
+    assert (out == src[96:1096]).all()
+    # a pending small upload reaches the stream on request
+    up = np.full(512, 0xab, np.uint8)
+    assert gpu.gpu_memcpy_h2d(d.ptr, up.ctypes.data, 512) == 0
+    gpu.anni_gpu_flush()
+    up[:] = 0                                            # staged at call time
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipStreamSynchronize.argtypes = [C.c_void_p]
+    assert hip.hipStreamSynchronize(gpu.anni_gpu_stream()) == 0       # the caller's own wait
+    got = np.zeros(512, np.uint8)
+    hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+    assert hip.hipMemcpy(got.ctypes.data, d.ptr, 512, 2) == 0          # 2 = device to host
+    assert (got == 0xab).all()
+    opt.free()
+    d.free()
 
 
 def test_malloc_and_free_from_many_threads(gpu):

@@ -263,7 +263,26 @@ def test_reference_production_flow_on_this_backend(gpu, oracle):
     p = M.params()
     m, v = M.moments()
     assert same_bits(p, P) and same_bits(m, Mo) and same_bits(v, Vo)
-    M.close()
+    # the consumer side of the twin flat (half_wt_get's flat branch, gpu_cuda.cu:2018-2034): after
+    # the steps of the unchanged caller, the slice served for every matrix is bf16 RNE of its weights
+    d_param, d_twin = M.device_flats()
+    assert d_param and d_twin
+    assert gpu.anni_gpu_bf16_twin_of(d_param, n) == d_twin
+    for off, cnt, is_mat in segs:
+        if not is_mat:
+            continue
+        served = gpu.anni_gpu_bf16_twin_of(d_param + 4 * off, cnt)
+        assert served == d_twin + 2 * off
+        got = np.empty(cnt, np.uint16)
+        assert gpu.gpu_memcpy_d2h(got.ctypes.data, served, 2 * cnt) == 0
+        assert (got == oracle.bf16_rne(P[off:off + cnt])).all(), off
+    assert gpu.anni_gpu_bf16_twin_of(d_param + 4, n) is None          # runs past the end of the flat
+    assert gpu.anni_gpu_bf16_twin_of(d_param - 4, 16) is None         # starts before it
+    other = gpu.gpu_malloc(1 << 20)
+    assert gpu.anni_gpu_bf16_twin_of(other, 1024) is None             # an activation: never a persistent twin
+    gpu.gpu_free(other)
+    M.close()                                                         # lm_adam_free: registration cleared, flats freed
+    assert gpu.anni_gpu_bf16_twin_of(d_param, 16) is None
     gpu.gpu_set_compute_prec(0)
     gpu.gpu_adam_set_weight_decay(0.0)
 

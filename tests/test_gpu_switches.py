@@ -32,6 +32,9 @@ def test_default_grid(gpu):
     assert run_child(ANNI_NT=0, ANNI_PIPE=0) == want
     assert run_child(ANNI_TILES_PER_WG=0) == want            # the resident grid
     assert run_child(ANNI_TILES_PER_WG=3, ANNI_PIPE=2) == want
+    # the norm's second stage taking the partials over with fences instead of atomic accesses:
+    # the same sum of squares (it is in the digests) and the same state, bit for bit
+    assert run_child(ANNI_FOLD="fence") == want
 
 
 def test_one_workgroup_per_cu_changeover_inside_every_workgroup(gpu):
