@@ -94,10 +94,60 @@ def adam_row(env, workload, size, grad_type, moment_type, n_params, warmup, step
     return row
 
 
+def _b(x):
+    return "true" if x else "false"
+
+
+def format_row(row):
+    """The row as the reference's writer prints it (lang/lm_bench.c:378-387 head, :586-608 body):
+    the same keys in the same order with the same printf conversions (%.0f, %.4f, %.1f, %.5f, %g,
+    %d, %ld); keys the reference does not have (cfg.phase, cfg.workload, params) follow the
+    reference's keys of their object.  A row parsed from a line of the reference's log prints
+    back as that line."""
+    m, c = row["model"], row["cfg"]
+    out = ('{"mode":"%s","git":"%s","dirty":%s,"backend":"%s","gpu":"%s","driver":"%s",'
+           '"vram_mb":%.0f,"busy":%s,"time":%d,"model":{"D":%d,"L":%d,"H":%d,"FF":%d}'
+           % (row["mode"], row["git"], _b(row["dirty"]), row["backend"], row["gpu"],
+              row["driver"], row["vram_mb"], _b(row["busy"]), row["time"], m["D"], m["L"], m["H"],
+              m["FF"]))
+    out += (',"cfg":{"V":%d,"B":%d,"B_req":%d,"T":%d,"prec":"%s","attn":"%s","graphs":%d,'
+            '"ckpt":%d,"offload":%d,"warmup":%d,"steps":%d,"lr":%g'
+            % (c["V"], c["B"], c["B_req"], c["T"], c["prec"], c["attn"], c["graphs"], c["ckpt"],
+               c["offload"], c["warmup"], c["steps"], c["lr"]))
+    for k in ("phase", "workload"):
+        if k in c:
+            out += ',"%s":"%s"' % (k, c[k])
+    ms = row["ms"]
+    out += ('},"ms":{"p10":%.4f,"p50":%.4f,"p90":%.4f,"mean":%.4f,"cv":%.4f},"tok_s":%.1f,'
+            '"tf_model":%.4f,"tf_hw":%.4f,"ceiling_tf":%.4f,"mfu":%.4f,"vram_peak_mb":%.0f,'
+            '"loss":[%.5f,%.5f],"loss_ok":%s'
+            % (ms["p10"], ms["p50"], ms["p90"], ms["mean"], ms["cv"], row["tok_s"],
+               row["tf_model"], row["tf_hw"], row["ceiling_tf"], row["mfu"], row["vram_peak_mb"],
+               row["loss"][0], row["loss"][1], _b(row["loss_ok"])))
+    if "phase_ms" in row:
+        ph = row["phase_ms"]
+        out += (',"phase_ms":{"fwd":%.4f,"loss":%.4f,"bwd":%.4f,"adam":%.4f}'
+                % (ph["fwd"], ph["loss"], ph["bwd"], ph["adam"]))
+    if "params" in row:
+        out += ',"params":%d' % row["params"]
+    return out + "}"
+
+
+IGNORED_CFG = ("warmup", "steps", "runs", "B_req", "lr")
+
+
+def compare_key(row):
+    """How the reference's scripts/bench_compare.py identifies a row (its key_of): mode, gpu,
+    model and cfg without warmup / steps / runs / B_req / lr, the two objects as sorted JSON."""
+    cfg = {k: v for k, v in row.get("cfg", {}).items() if k not in IGNORED_CFG}
+    return (row.get("mode"), row.get("gpu"), json.dumps(row.get("model", {}), sort_keys=True),
+            json.dumps(cfg, sort_keys=True))
+
+
 def append(path, row):
     """Appends the row as one line (the reference opens its log with "a", lm_bench.c:362-375)."""
     d = os.path.dirname(path)
     if d:
         os.makedirs(d, exist_ok=True)
     with open(path, "a", encoding="utf-8") as fp:
-        fp.write(json.dumps(row, separators=(",", ":")) + "\n")
+        fp.write(format_row(row) + "\n")

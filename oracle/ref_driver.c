@@ -15,6 +15,7 @@
 #include "lm_serialize.h"
 #include "lm_train.h"
 #include "layernorm.h"
+#include "lm_bench.h"
 
 typedef struct ref_adam {
 	lm_adam	opt;
@@ -332,4 +333,29 @@ double ref_step_lr(double base_lr, int step, int warmup, int decay_steps,
 	lm_train_set_lr_sched_from(0);
 	lm_train_set_lr_schedule(0, 0, "none");
 	return lr;
+}
+
+/*
+** The reference's own bench harness, `anni lm bench step --profile --json FILE`
+** (lang/lm_bench.c:619-643): one packed training step per iteration on whatever backend is
+** linked, one JSON line appended to `json`.  Returns lm_bench_step's result (0 done, 1 loss
+** check failed, 2 refused: its harness refuses to run on the CPU stub).
+*/
+int ref_bench_step(const char *json, int B, int T, int vocab, int warmup, int steps)
+{
+	lm_bench_cfg cfg;
+
+	lm_bench_cfg_defaults(&cfg);
+	cfg.B = B;
+	cfg.T = T;
+	cfg.vocab = vocab;
+	cfg.prec = LM_BENCH_FP32;
+	cfg.graphs = 0;
+	cfg.warmup = warmup;
+	cfg.steps = steps;
+	cfg.profile = 1;
+	cfg.ceiling = 0;
+	cfg.allow_busy = 1;
+	cfg.json = json;
+	return lm_bench_step(&cfg);
 }

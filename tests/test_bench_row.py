@@ -48,25 +48,76 @@ def test_row_has_every_key_of_the_reference_row():
     assert bench_row.adam_row(ENV, "1p4b-fp8", "1p4b", 2, 0, 1, 0, [1.0], 3e-4, 0, False)["loss_ok"] is False
 
 
-def compare_key(row):
-    """How the reference's comparison script identifies a row: mode, gpu, model, cfg without
-    warmup / steps / runs / B_req / lr."""
-    cfg = {k: v for k, v in row["cfg"].items() if k not in ("warmup", "steps", "runs", "B_req", "lr")}
-    return (row["mode"], row["gpu"], json.dumps(row["model"], sort_keys=True),
-            json.dumps(cfg, sort_keys=True))
+def _fixtures():
+    import os
+    from helpers import GOLDEN
+    line = open(os.path.join(GOLDEN, "bench_row_ref.jsonl")).read().rstrip("\n")
+    keys = json.load(open(os.path.join(GOLDEN, "bench_row_keys.json")))
+    return line, keys
 
 
-def test_rows_of_two_runs_match_and_never_match_a_whole_step_row(tmp_path):
+def _sample_row():
+    import importlib.util
+    import os
+    from helpers import GOLDEN
+    spec = importlib.util.spec_from_file_location("make_bench_row",
+                                                  os.path.join(GOLDEN, "make_bench_row.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod.sample_row()
+
+
+def test_writer_reproduces_the_line_the_references_writer_wrote():
+    """tests/golden/bench_row_ref.jsonl is the line the reference's own lm_bench_step appended when
+    its real training step ran on this backend (make_bench_row.py --row).  Parsed and printed back
+    by format_row it must be that line, byte for byte: key order, nesting, %.4f / %.1f / %.5f /
+    %.0f / %g conversions."""
+    line, _keys = _fixtures()
+    ref = json.loads(line)
+    assert bench_row.format_row(ref) == line
+    # and our own rows carry the reference's keys in the reference's order, extras behind them
+    ours = _sample_row()
+    printed = json.loads(bench_row.format_row(ours))
+    assert [k for k in printed if k in ref] == list(ref)
+    assert list(printed)[len(ref):] == ["params"]
+    assert list(printed["cfg"])[:len(ref["cfg"])] == list(ref["cfg"])
+    assert list(printed["cfg"])[len(ref["cfg"]):] == ["phase", "workload"]
+    for k in ("model", "ms", "phase_ms"):
+        assert list(printed[k]) == list(ref[k])
+    assert printed == json.loads(json.dumps(ours))       # nothing lost on the way
+    # number formats of our values as the reference prints such values
+    text = bench_row.format_row(ours)
+    assert '"ms":{"p10":3.1999,"p50":3.2101,' in text and '"lr":0.0003,' in text
+    assert '"mfu":-1.0000,' in text and '"loss":[-1.00000,-1.00000]' in text
+    assert '"vram_mb":294896,' in text and '"tok_s":0.0,' in text
+
+
+def test_compare_key_is_the_references_key_of():
+    """bench_row.compare_key against the keys that the reference's scripts/bench_compare.py itself
+    derived (make_bench_row.py --keys imported it in the build container) for the reference-written
+    row and for a row of ours."""
+    line, keys = _fixtures()
+    ref = json.loads(line)
+    assert list(bench_row.compare_key(ref)) == keys["ref_row_key"]
+    ours = _sample_row()
+    assert json.loads(json.dumps(ours)) == keys["sample_row"]    # the row the key was recorded for
+    assert list(bench_row.compare_key(ours)) == keys["sample_row_key"]
+    assert sorted(bench_row.IGNORED_CFG) == keys["ignored_cfg"]
+    # a whole-step row of the same gpu and model is another key: the two kinds never match
+    whole = dict(ref, gpu=ours["gpu"], model=ours["model"])
+    assert list(bench_row.compare_key(whole)) == keys["whole_step_row_same_gpu_model_key"]
+    assert bench_row.compare_key(whole) != bench_row.compare_key(ours)
+    # the scored metric of a step row is ms.p50, lower is better, and ours is a positive number
+    assert keys["step_metric"] == [["ms", "p50"], False]
+    assert keys["sample_row_metric"] == ours["ms"]["p50"] > 0
+
+
+def test_rows_of_two_runs_match(tmp_path):
     a = bench_row.adam_row(ENV, "555m", "555m", 0, 0, 555848096, 3, [3.4] * 10, 3e-4, 98000.0, True)
     b = bench_row.adam_row(ENV, "555m", "555m", 0, 0, 555848096, 5, [3.3] * 20, 1e-4, 98000.0, True)
-    assert compare_key(a) == compare_key(b)             # warmup / steps / lr do not matter
+    assert bench_row.compare_key(a) == bench_row.compare_key(b)   # warmup / steps / lr do not matter
     c = bench_row.adam_row(ENV, "555m-bf16", "555m", 1, 1, 555848096, 3, [2.3] * 8, 3e-4, 1.0, True)
-    assert compare_key(c) != compare_key(a)
-    whole = json.loads(json.dumps(a))
-    del whole["cfg"]["phase"], whole["cfg"]["workload"]  # what a row of the reference's own bench has
-    assert compare_key(whole) != compare_key(a)
-    # the scored metric is ms.p50, which must be a positive number
-    assert isinstance(a["ms"]["p50"], float) and a["ms"]["p50"] > 0
+    assert bench_row.compare_key(c) != bench_row.compare_key(a)
     path = str(tmp_path / "bench" / "run.jsonl")
     bench_row.append(path, a)
     bench_row.append(path, b)
