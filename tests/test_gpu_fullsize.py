@@ -378,3 +378,50 @@ def test_more_than_2_to_31_elements(gpu, oracle, mode):
         assert not opt.download("m", k, at).any() and not opt.download("v", k, at).any()
         assert not opt.download("grad", k, at).any()
     opt.free()
+
+
+@pytest.mark.parametrize("ballast_gib", [150, 262])
+def test_arena_creation_with_most_of_the_memory_taken(gpu, oracle, ballast_gib):
+    """anni_adam_create does not assume an empty GPU: with 150 GiB held by someone else the search
+    for the second half still finds memory of another section or ends without one, with 262 GiB
+    held (about 20 GiB left) there is nothing to search; either way the arena is created at its
+    exact size, a step gives the oracle's bits, and everything is returned afterwards."""
+    import ctypes as C
+    gpu.gpu_device_sync()
+    fr0, tt = C.c_size_t(0), C.c_size_t(0)
+    assert gpu.gpu_mem_info(C.byref(fr0), C.byref(tt)) == 0
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+    hip.hipFree.argtypes = [C.c_void_p]
+    blocks = []
+    left = ballast_gib - (tt.value - fr0.value) // (1 << 30)        # what is in use already counts
+    while left > 0:
+        p = C.c_void_p()
+        take = min(left, 16)
+        assert hip.hipMalloc(C.byref(p), take << 30) == 0, (ballast_gib, left)
+        blocks.append(p)
+        left -= take
+    opt, tensors, segs, mask = setup(gpu, "185m", skip_nonfinite=True)
+    n = opt.n
+    assert opt.split and opt.arena_bytes <= opt.resident_bytes + (16 << 20)
+    print("ballast %d GiB: apart ratio %.3f" % (ballast_gib, opt.apart_ratio), flush=True)
+    P, M, V = opt.download("param"), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True,
+                      tensors=segs, threads=THREADS, simd=oracle.cpu_simd())
+    assert gpu.anni_fill_normal_f32(opt.o.d_grad, n, 7, 300, 0.0, 1e-3) == 0
+    g = opt.download("grad")
+    gs = 1.7 / (math.sqrt(n) * 1e-3)
+    opt.step_scaled(3e-4, gs)
+    st = opt.sync_stats()
+    O.step(P, g, M, V, 3e-4, gs, sumsq_override=st.last_sumsq)
+    assert st.last_clipped == 1 == O.o.last_clipped
+    assert same_bits(opt.download("param"), P) and same_bits(opt.download("m"), M)
+    assert same_bits(opt.download("v"), V)
+    assert (opt.download("twin")[mask] == oracle.bf16_rne(P)[mask]).all()
+    opt.free()
+    for p in blocks:
+        assert hip.hipFree(p) == 0
+    gpu.gpu_device_sync()
+    fr1 = C.c_size_t(0)
+    assert gpu.gpu_mem_info(C.byref(fr1), C.byref(tt)) == 0
+    assert abs(fr1.value - fr0.value) <= 64 << 20
