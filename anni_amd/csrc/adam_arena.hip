@@ -16,6 +16,7 @@
 #include <vector>
 #include "adam_kernels.h"
 #include "anni_adam.h"
+#include "anni_bench.h"
 #include "anni_gpu.h"
 #include "backend_state.h"
 #include "placement.h"

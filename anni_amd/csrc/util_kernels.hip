@@ -9,6 +9,7 @@
 #include <stdint.h>
 #include "adam_kernels.h"
 #include "anni_adam.h"
+#include "anni_bench.h"
 #include "backend_state.h"
 
 namespace anni {

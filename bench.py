@@ -378,6 +378,104 @@ def ckpt_leg(L, size="555m"):
     return out
 
 
+def sections_leg(L, n=555848096, region_gib=16):
+    """How device memory is organised, measured: free memory is taken as physical blocks of 16 GiB
+    (HIP virtual memory management: each a naturally aligned block while memory is free, handed
+    out from the highest address down), each mapped at its own address; the flat-ABI update
+    (gpu_adam_step_dev_bf16, all-zero state, which it leaves zero) then runs with its five flats
+    in chosen blocks.  Reports the update's GB/s for every window of five consecutive blocks, the
+    runs of blocks ("sections") those windows reveal, and for a few placements."""
+    hip = C.CDLL("libamdhip64.so")
+
+    class Loc(C.Structure):
+        _fields_ = [("type", C.c_int), ("id", C.c_int)]
+
+    class Prop(C.Structure):                      # hipMemAllocationProp
+        _fields_ = [("type", C.c_int), ("handle_type", C.c_int), ("location", Loc),
+                    ("win32", C.c_void_p), ("compression", C.c_ubyte), ("rdma", C.c_ubyte),
+                    ("usage", C.c_ushort)]
+
+    class Access(C.Structure):                    # hipMemAccessDesc
+        _fields_ = [("location", Loc), ("flags", C.c_int)]
+    hip.hipMemCreate.argtypes = [C.POINTER(C.c_void_p), C.c_size_t, C.POINTER(Prop), C.c_ulonglong]
+    hip.hipMemAddressReserve.argtypes = [C.POINTER(C.c_void_p), C.c_size_t, C.c_size_t, C.c_void_p,
+                                         C.c_ulonglong]
+    hip.hipMemMap.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_ulonglong]
+    hip.hipMemSetAccess.argtypes = [C.c_void_p, C.c_size_t, C.POINTER(Access), C.c_size_t]
+    hip.hipMemUnmap.argtypes = [C.c_void_p, C.c_size_t]
+    hip.hipMemRelease.argtypes = [C.c_void_p]
+    hip.hipMemAddressFree.argtypes = [C.c_void_p, C.c_size_t]
+    prop = Prop(1, 0, Loc(1, 0), None, 0, 0, 0)   # pinned device memory of device 0
+    acc = Access(Loc(1, 0), 3)                    # read-write
+    size = region_gib << 30
+    fr, tt = C.c_size_t(0), C.c_size_t(0)
+    blocks = []
+    while L.gpu_mem_info(C.byref(fr), C.byref(tt)) == 0 and fr.value >= size + (3 << 30):
+        h, va = C.c_void_p(), C.c_void_p()
+        if hip.hipMemCreate(C.byref(h), size, C.byref(prop), 0) != 0:
+            break
+        assert hip.hipMemAddressReserve(C.byref(va), size, 0, None, 0) == 0
+        assert hip.hipMemMap(va, size, 0, h, 0) == 0
+        assert hip.hipMemSetAccess(va, size, C.byref(acc), 1) == 0
+        assert L.gpu_memset(va.value, 0, 10 << 30) == 0       # what the flats below touch
+        blocks.append((h, va.value))
+    L.gpu_device_sync()
+    K = len(blocks)
+    L.gpu_set_compute_prec(1)
+    L.gpu_adam_set_weight_decay(0.1)
+
+    def run(places, reps=4):
+        """places: (block, offset GiB) of p, m, v, twin, g -> GB/s of algorithmic traffic."""
+        p, m, v, tw, g = [blocks[b][1] + int(off * (1 << 30)) for b, off in places]
+        args = (p, tw, g, m, v, n, 1e-3, 0.9, 0.95, 1e-8, 3, 1.0)
+        assert L.gpu_adam_step_dev_bf16(*args) == 0
+        L.gpu_device_sync()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            L.gpu_adam_step_dev_bf16(*args)
+        L.gpu_device_sync()
+        return round(n * 34 * reps / (time.perf_counter() - t0) / 1e9, 1)
+    out = {"blocks_of_GiB": region_gib, "blocks": K, "params": n,
+           "free_GiB_before": round((fr.value + K * size) / (1 << 30), 1)}
+    win = [run([(b + i, 0) for i in range(5)]) for b in range(K - 4)]
+    out["window_of_five_consecutive_blocks_GBps"] = win
+    # a window inside one section is slow; the first fast window b means a boundary behind block b+3
+    cut = (max(win) + min(win)) / 2
+    sec, cur, b = [0] * K, 0, 0
+    bounds = []
+    while b < K - 4:
+        if win[b] > cut:
+            bounds.append(b + 4)
+            b += 4
+        else:
+            b += 1
+    for i in range(K):
+        sec[i] = sum(1 for x in bounds if i >= x)
+    out["section_of_block"] = sec
+    members = [[i for i in range(K) if sec[i] == s] for s in range(max(sec) + 1)]
+    out["blocks_per_section"] = [len(m) for m in members]
+    if len(members) >= 3 and min(len(m) for m in members[:3]) >= 5:
+        A, B_, C_ = members[0], members[1], members[2]
+        out["placements_GBps"] = {
+            "all five flats in ONE block (3 GiB apart)": run([(A[0], 3 * i) for i in range(5)]),
+            "five blocks of section A": run([(A[i], 0) for i in range(5)]),
+            "five blocks of section B, not consecutive": run([(B_[i], 0) for i in (0, 1, 3, 4, 5)] if len(B_) > 5 else [(B_[i], 0) for i in range(5)]),
+            "p m | v twin g (two sections, as the split arena)": run([(A[0], 0), (A[1], 0), (B_[0], 0), (B_[1], 0), (B_[2], 0)]),
+            "p m | v twin g, each side inside ONE block": run([(A[0], 0), (A[0], 4), (B_[0], 0), (B_[0], 4), (B_[0], 7)]),
+            "p m v twin | g": run([(A[0], 0), (A[1], 0), (A[2], 0), (A[3], 0), (B_[0], 0)]),
+            "p | m v twin g": run([(A[0], 0), (B_[0], 0), (B_[1], 0), (B_[2], 0), (B_[3], 0)]),
+            "p g | m v | twin (three sections)": run([(A[0], 0), (B_[0], 0), (B_[1], 0), (C_[0], 0), (A[1], 0)]),
+            "p twin g | m v": run([(A[0], 0), (B_[0], 0), (B_[1], 0), (A[1], 0), (A[2], 0)]),
+        }
+    L.gpu_set_compute_prec(0)
+    L.gpu_adam_set_weight_decay(0.0)
+    for h, va in blocks:
+        hip.hipMemUnmap(va, size)
+        hip.hipMemRelease(h)
+        hip.hipMemAddressFree(va, size)
+    return out
+
+
 def ceilings(L, nbytes=8 << 30):
     """What this box delivers to the simplest kernels of the library: write-only (fill), copy
     (16-byte vectors, read + write) and read-only (the sum of squares), for comparison with the
@@ -442,6 +540,9 @@ def main():
                     help="only time the optimizer block of a checkpoint written from / read into the arena")
     ap.add_argument("--ceilings", action="store_true",
                     help="only measure write-only, copy and read-only throughput of the box")
+    ap.add_argument("--sections", action="store_true",
+                    help="only map free device memory as 16 GiB physical blocks and time the update with its "
+                         "flats in chosen blocks: shows the three 96 GiB sections the placement is about")
     ap.add_argument("--colsum", type=int, default=0, metavar="ROWS",
                     help="only time the bias / LayerNorm gradient column sums over ROWS token rows")
     ap.add_argument("--reference-caller-only", action="store_true",
@@ -478,6 +579,9 @@ def main():
         return
     if a.ceilings:
         print(json.dumps({"ceilings": ceilings(L)}))
+        return
+    if a.sections:
+        print(json.dumps({"sections": sections_leg(L)}))
         return
     if a.colsum:
         print(json.dumps({"colsum_add": colsum_leg(L, a.colsum)}))

@@ -242,37 +242,11 @@ void	anni_gpu_set_stream(void *hip_stream);
 */
 void	anni_gpu_flush(void);
 
-/*
-** Reads the kernels' tuning switches (ANNI_TILES_PER_WG, ANNI_KEEP_MB, ANNI_REVERSE, ANNI_PIPE,
-** ANNI_NT, ANNI_BLOCKS_PER_CU) from the environment again; without this call they are read once,
-** on first use.  For sweeps that compare settings on one arena inside one process
-** (`bench.py --sweep`); results never depend on them.  No counterpart in the reference.
-*/
-void	anni_gpu_reload_switches(void);
-
 /* Name and architecture of the current device and the HIP driver version: what the reference's bench row records from nvidia-smi (lang/lm_bench.c:287-316). */
 int	anni_gpu_device_info(char *name, size_t cap, int *driver_version);
 
-/*
-** Times `count` back-to-back steps with HIP events recorded on the compute
-** stream: per step, the gradient flat grads[i % n_grads] is bound (NULL array =
-** keep the bound one), lr[i] and grad_scale[i] are used.  ms_total receives the
-** elapsed time of the whole run, ms_sumsq / ms_update (may be NULL) the summed
-** durations of the two kernels.  Allocates nothing on the device.
-*/
-int	anni_adam_time_steps(anni_adam *opt, int count, void *const *grads, int n_grads,
-		const double *lr, const double *grad_scale, float *ms_total,
-		float *ms_sumsq, float *ms_update);
-/* Summed duration of the E4M3 twin launches of the last anni_adam_time_steps run that asked for per-kernel times. */
-float	anni_adam_timed_derived_ms(const anni_adam *opt);
-
 /* ---- producers either side of the step (device utilities) ---------------- */
 
-/* x[i] = mean + std * N(0,1), counter-based (seed, stream, i): same values for any launch shape. */
-int	anni_fill_normal_f32(float *d_x, int64_t n, uint64_t seed, uint64_t stream,
-		float mean, float std);
-/* Plain 16-byte-vector copy kernel of nbytes (a multiple of 16, 16-byte aligned): reads and writes exactly nbytes. */
-int	anni_copy_bytes(void *d_dst, const void *d_src, size_t nbytes);
 /* dst = bf16(src) round to nearest even (num/gpu_cuda.cu:1497-1513). */
 int	anni_f32_to_bf16(void *d_dst, const float *d_src, int64_t n);
 /*
