@@ -43,17 +43,15 @@ struct Elem {
 ** a / b for a step constant b whose correctly rounded reciprocal rb the host supplies:
 ** q = a*rb, then one exact residual a - b*q folded back.  The result is a/b rounded to
 ** nearest unless a/b lies within ~2^-52 ulp of a rounding boundary (then it may be the
-** other neighbour): about one quotient in 2^52.  A quotient that is not finite (a moment that
-** overflowed to infinity, a NaN) is returned as it is, as the division gives it -- its residual
-** would be inf - inf.  Used only where the update is bound by arithmetic (narrow storage
-** types); the all-f32 mode keeps the IEEE division.
+** other neighbour): about one quotient in 2^52.  Not for an infinite a: the residual would be
+** inf - inf (adam_elem sends those to the IEEE division).  Used only where the update is bound
+** by arithmetic (narrow storage types); the all-f32 mode keeps the IEEE division.
 */
 __device__ __forceinline__ double div_by_const(double a, double b, double rb)
 {
 	const double q = a * rb;
-	const double r = __builtin_fma(__builtin_fma(-b, q, a), rb, q);
 
-	return __builtin_isfinite(q) ? r : q;
+	return __builtin_fma(__builtin_fma(-b, q, a), rb, q);
 }
 
 /*
@@ -66,11 +64,35 @@ __device__ __forceinline__ Elem adam_elem(float p, float g, float m, float v, do
 {
 	Elem r;
 	const double x = (double)g * gs;
+	double mhat, vhat;
 
 	r.m = (float)(c.beta1 * (double)m + c.omb1 * x);
 	r.v = (float)(c.beta2 * (double)v + (c.omb2 * x) * x);
-	const double mhat = FASTDIV ? div_by_const((double)r.m, c.bc1, c.rbc1) : (double)r.m / c.bc1;
-	const double vhat = FASTDIV ? div_by_const((double)r.v, c.bc2, c.rbc2) : (double)r.v / c.bc2;
+	if (FASTDIV) {
+		mhat = div_by_const((double)r.m, c.bc1, c.rbc1);
+		vhat = div_by_const((double)r.v, c.bc2, c.rbc2);
+		/*
+		** A moment that overflowed to infinity (or is NaN): the host loop divides it all the same
+		** -- inf / bc2 = inf, sqrt(inf) = inf, the step is 0 -- while the residual above gives
+		** NaN.  |m| + v is finite exactly when both are (or spuriously not, next to the largest
+		** float: harmless); the wavefront leaves the fast path only when a lane needs to.
+		*/
+		const bool odd = !__builtin_isfinite(__builtin_fabsf(r.m) + r.v);
+
+		if (__builtin_expect(__builtin_amdgcn_ballot_w64(odd) != 0, 0)) {
+			float fm = r.m, fv = r.v;
+
+			/* keeps the two divisions inside this block (they would be hoisted and selected otherwise) */
+			asm volatile("" : "+v"(fm), "+v"(fv));
+			if (odd) {
+				mhat = (double)fm / c.bc1;
+				vhat = (double)fv / c.bc2;
+			}
+		}
+	} else {
+		mhat = (double)r.m / c.bc1;
+		vhat = (double)r.v / c.bc2;
+	}
 	r.p = (float)((double)p - (c.lr * mhat) / (sqrt(vhat) + c.eps));
 	if (decay)
 		r.p = (float)((double)r.p - c.lr_wd * (double)r.p);

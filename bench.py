@@ -613,9 +613,11 @@ def main():
     n_params = sum(t[1] for t in tensors)
     slot_bytes = -(-n_params * ELEM[gt] // (2 << 20)) * (2 << 20)
     n_slots = min(total, max(4, (32 << 30) // slot_bytes))
+    t_create = time.perf_counter()
     opt = LmAdam(tensors, grad_type=gt, moment_type=mt, twins=True, skip_nonfinite=True,
                  grad_slots=n_slots, layout={"auto": 0, "compact": 1, "split": 2}[a.layout],
                  beta2=0.95, weight_decay=0.1, grad_clip=1.0)
+    t_create = (time.perf_counter() - t_create) * 1e3
     n = opt.n
     assert L.anni_fill_normal_f32(opt.o.d_param, n, 20260101, 1, 0.0, 0.02) == 0
     if a.derived:
@@ -718,7 +720,8 @@ def main():
                    "placement_apart_ratio": round(opt.apart_ratio, 3),
                    "placement_probe_GBps": round(opt.probe_gbps, 1),
                    "arena_bytes": opt.arena_bytes, "resident_bytes": opt.resident_bytes,
-                   "grad_slots": n_slots, "launches_per_step": 2},
+                   "grad_slots": n_slots, "arena_create_ms": round(t_create, 1),
+                   "launches_per_step": 2},
         "params_per_s": round(n / (ms_step * 1e-3), 1),
         "pct_of_hbm_peak": round(100.0 * step_gbps / HBM_PEAK_GBPS, 2),
         "event_ms_per_step": round(ev_ms / a.steps, 4),
