@@ -114,9 +114,9 @@ template <bool PROD> struct CsRows { static constexpr int n = 64; };
 /*
 ** Rows FIRST .. FIRST + COUNT - 1 of a chunk of the lane's column into registers, as raw buffer loads: the
 ** descriptor (scalar registers) starts at the chunk's first row, the row offset is a scalar, the
-** lane supplies only its constant column offset -- no vector arithmetic per load.  A chunk that
-** runs past the matrix reads its last valid row again for the rows beyond it (those registers are
-** never added): the scalar row index is clamped, one scalar minimum per load, so every address
+** lane supplies only its constant column offset -- no vector arithmetic per load.  The one chunk
+** of a column that runs past the matrix reads its last valid row again for the rows beyond it
+** (those registers are never added): there the scalar row index is clamped, so every address
 ** lies inside the matrix by construction.  (The descriptor's range check is not relied on for
 ** this: it compares the vector offset only, the scalar offset takes no part in it.)  A select on
 ** a loaded value instead would make the wavefront wait for the load on the spot.
@@ -140,6 +140,18 @@ __device__ __forceinline__ void colsum_fetch(float (&rx)[CsRows<PROD>::n], float
 	    (void *)((PROD ? y : x) + r0 * cols), 0, (int)span, 0x00020000);
 	const uint32_t pitch = (uint32_t)cols * (uint32_t)sizeof(float);
 
+	if (rows_left >= kCsRows) {
+		/* a whole chunk (all but the last one of a column): the row offsets are multiples of the pitch */
+#pragma unroll
+		for (int i = FIRST; i < FIRST + COUNT; i++) {
+			rx[i] = __builtin_bit_cast(float,
+			    __builtin_amdgcn_raw_buffer_load_b32(bx, (int)col_bytes, (int)(i * pitch), 0));
+			if (PROD)
+				ry[i] = __builtin_bit_cast(float,
+				    __builtin_amdgcn_raw_buffer_load_b32(by, (int)col_bytes, (int)(i * pitch), 0));
+		}
+		return;
+	}
 #pragma unroll
 	for (int i = FIRST; i < FIRST + COUNT; i++) {
 		const uint32_t row = (uint32_t)i < last ? (uint32_t)i : last;
