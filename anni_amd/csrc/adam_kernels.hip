@@ -1218,6 +1218,7 @@ struct Switches {
 	int	keep_mb;	/* ANNI_KEEP_MB: how much of the gradients' tail the sum of squares leaves in the memory-side cache */
 	int	pipe;		/* ANNI_PIPE=0: narrow storage modes on the plain kernel; 2: the all-f32 mode pipelined too */
 	int	tiles_per_wg;	/* ANNI_TILES_PER_WG: tiles per workgroup of the update; 0 = the resident grid; -1 = the default */
+	int	sumsq_per_cu;	/* ANNI_SUMSQ_PER_CU: workgroups per compute unit of the sum of squares; 0 = the default */
 	int	fold_fence;	/* ANNI_FOLD=fence: the norm's second stage takes the partials over with fences (see sumsq_finish) */
 };
 static Switches g_sw;
@@ -1230,6 +1231,7 @@ void reload_switches(void)
 	g_sw.keep_mb = env_int("ANNI_KEEP_MB", 256, 0, 1 << 20);
 	g_sw.pipe = env_int("ANNI_PIPE", 1, 0, 2);
 	g_sw.tiles_per_wg = env_int("ANNI_TILES_PER_WG", -1, -1, 1 << 20);
+	g_sw.sumsq_per_cu = env_int("ANNI_SUMSQ_PER_CU", 0, 0, 32);
 	{
 		const char *e = getenv("ANNI_FOLD");
 
@@ -1334,9 +1336,23 @@ int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *parti
 	    : f.grad_type == kBF16 ? SumsqChunk<kBF16>::kElems : SumsqChunk<kFP8>::kElems;
 	const int64_t n_chunks = (f.n + chunk_elems - 1) / chunk_elems;
 
-	grid = grid_for(f.n);
-	if (grid > n_chunks)
-		grid = (int)n_chunks;
+	{
+		/*
+		** Workgroups of the sum, resident as a whole.  Float gradients: two per compute unit
+		** (0.327 against 0.337 ms for eight at 555M, measured inside one process; one is too few,
+		** 0.444).  bf16 and E4M3 gradients do more arithmetic per byte and want the usual eight
+		** (two: +25 - 35 %).
+		*/
+		const int per_cu = sw().sumsq_per_cu ? sw().sumsq_per_cu
+		    : f.grad_type == kF32 ? 2 : sw().blocks_per_cu;
+		int64_t g = (int64_t)cu_count() * per_cu;
+
+		if (g > kMaxPartials)
+			g = kMaxPartials;
+		if (g > n_chunks)
+			g = n_chunks;
+		grid = g < 1 ? 1 : (int)g;
+	}
 	a.g = f.g;
 	a.n = f.n;
 	a.segs = f.segs;

@@ -41,7 +41,7 @@ def test_one_workgroup_per_cu_changeover_inside_every_workgroup(gpu):
     """256 workgroups over ~2200 tiles: each one takes 8 or 9 tiles, and with 5 MiB kept the
     changeover from streaming to ordinary loads falls inside every workgroup's run (after one round
     of the grid for fp8 codes)."""
-    want = run_child(ANNI_BLOCKS_PER_CU=1, ANNI_KEEP_MB=0)
-    assert run_child(ANNI_BLOCKS_PER_CU=1, ANNI_KEEP_MB=5) == want
-    assert run_child(ANNI_BLOCKS_PER_CU=1, ANNI_KEEP_MB=3, ANNI_REVERSE=0) == want
-    assert run_child(ANNI_BLOCKS_PER_CU=1, ANNI_KEEP_MB=100000) == want
+    want = run_child(ANNI_BLOCKS_PER_CU=1, ANNI_SUMSQ_PER_CU=1, ANNI_KEEP_MB=0)
+    assert run_child(ANNI_BLOCKS_PER_CU=1, ANNI_SUMSQ_PER_CU=1, ANNI_KEEP_MB=5) == want
+    assert run_child(ANNI_BLOCKS_PER_CU=1, ANNI_SUMSQ_PER_CU=1, ANNI_KEEP_MB=3, ANNI_REVERSE=0) == want
+    assert run_child(ANNI_BLOCKS_PER_CU=1, ANNI_SUMSQ_PER_CU=1, ANNI_KEEP_MB=100000) == want
