@@ -1175,15 +1175,14 @@ __global__ __launch_bounds__(kThreads) void fill_bytes_kernel(uint8_t *dst, uint
 	/* [0, head) bytes up to 16-byte alignment, n16 aligned 16-byte words, then the rest. */
 	for (size_t i = gid; i < head; i += stride)
 		dst[i] = (uint8_t)pattern;
-	/* one contiguous slice per workgroup: measured 5.8 TB/s against 5.2 for a grid-stride walk */
-	{
-		const size_t per = (n16 + gridDim.x - 1) / gridDim.x;
-		const size_t first = (size_t)blockIdx.x * per;
-		const size_t last = first + per < n16 ? first + per : n16;
-
-		for (size_t i = first + threadIdx.x; i < last; i += kThreads)
-			*(u32x4 *)(dst + head + i * 16) = w;
-	}
+	/*
+	** Word i goes to lane i mod (all lanes of the grid): with ONE workgroup per compute unit the
+	** chip then writes one contiguous MiB at a time, every workgroup always the same 4 KiB of it --
+	** measured 6.4 - 6.5 TB/s, what the runtime's own fill reaches, against 5.8 - 6.0 for any grid
+	** of more workgroups (512: 5.3, 2048: 4.9) and for one contiguous slice or tile per workgroup.
+	*/
+	for (size_t i = gid; i < n16; i += stride)
+		*(u32x4 *)(dst + head + i * 16) = w;
 	for (size_t i = head + n16 * 16 + gid; i < nbytes; i += stride)
 		dst[i] = (uint8_t)pattern;
 }
@@ -1677,8 +1676,15 @@ int launch_fill_bytes(hipStream_t st, void *dst, int value, size_t nbytes)
 	if (head > nbytes)
 		head = nbytes;
 	n16 = (nbytes - head) / 16;
-	hipLaunchKernelGGL(fill_bytes_kernel, dim3(helper_grid((int64_t)n16 + 16)), dim3(kThreads),
-	    0, st, (uint8_t *)dst, pattern, nbytes, head, n16);
+	{
+		/* large fills: one workgroup per compute unit (see the kernel) */
+		int grid = helper_grid((int64_t)n16 + 16);
+
+		if (grid > cu_count())
+			grid = cu_count();
+		hipLaunchKernelGGL(fill_bytes_kernel, dim3(grid), dim3(kThreads), 0, st, (uint8_t *)dst,
+		    pattern, nbytes, head, n16);
+	}
 	return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
