@@ -53,7 +53,6 @@ int	gpu_ce_bias_fused(void) ANSWER(0)
 int	gpu_ce_bf16_delta_done(const ann_real *) NOT_HERE
 int	gpu_ce_nll_rows(const ann_real *, const int *, int, int, float *) NOT_HERE
 int	gpu_posenc_add_packed(ann_real *, int, int, int) NOT_HERE
-int	gpu_mat_col_sum_add(ann_real *, const ann_real *, int, int) NOT_HERE
 int	gpu_relu_backward(ann_real *, const ann_real *, int) NOT_HERE
 int	gpu_ffn_relu_bwd_fused(mat *, const mat *, ann_real *) NOT_HERE
 int	gpu_act_bf16_only(const mat *) ANSWER(0)

@@ -7,8 +7,10 @@
 */
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <mutex>
 #include "adam_kernels.h"
 #include "anni_adam.h"
+#include "anni_gpu.h"
 #include "anni_bench.h"
 #include "backend_state.h"
 
@@ -393,6 +395,46 @@ int anni_colsum_add(float *d_acc, const float *d_x, const float *d_y, int64_t ro
 	job.rows = rows;
 	job.cols = cols;
 	return anni_colsum_add_batch(&job, 1);
+}
+
+int gpu_mat_col_sum_add(ann_real *db_host, const ann_real *x, int rows, int cols)
+{
+	static std::mutex mu;			/* one accumulator, grown on demand */
+	static float *d_acc;
+	static int d_acc_cols;
+	hipPointerAttribute_t attr;
+	hipStream_t st;
+	int rc = -1;
+
+	if (!db_host || !x || rows <= 0 || cols <= 0 || !device_ready())
+		return -1;
+	if (hipPointerGetAttributes(&attr, x) != hipSuccess || attr.type != hipMemoryTypeDevice) {
+		(void)hipGetLastError();
+		return -1;			/* a host matrix: the caller's own loop */
+	}
+	std::lock_guard<std::mutex> lk(mu);
+
+	if (cols > d_acc_cols) {
+		void *p = nullptr;
+
+		if (!hip_ok(hipMalloc(&p, (size_t)cols * sizeof(float)), "colsum hipMalloc")) {
+			(void)hipGetLastError();
+			return -1;
+		}
+		if (d_acc)
+			(void)hipFree(d_acc);
+		d_acc = (float *)p;
+		d_acc_cols = cols;
+	}
+	st = compute_stream();
+	if (hip_ok(hipMemcpyAsync(d_acc, db_host, (size_t)cols * sizeof(float), hipMemcpyHostToDevice, st),
+	    "colsum h2d")
+	    && anni_colsum_add(d_acc, x, nullptr, rows, cols) == 0
+	    && hip_ok(hipMemcpyAsync(db_host, d_acc, (size_t)cols * sizeof(float), hipMemcpyDeviceToHost,
+	    compute_stream()), "colsum d2h")
+	    && hip_ok(sync_stream_and_deliver(), "colsum sync"))
+		rc = 0;
+	return rc;
 }
 
 int anni_fp8_quantize(void *d_q, float *d_scale, const float *d_src, int64_t n)

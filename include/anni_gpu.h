@@ -104,6 +104,19 @@ unsigned	gpu_param_epoch(void);
 */
 const void	*anni_gpu_bf16_twin_of(const ann_real *fp32_dev, size_t n);
 
+/*
+** num/gpu.h:195-199 -- db_host[cols] += column sums of the rows x cols matrix x (a bias gradient,
+** lang/ffn.c:298,355).  Served when x is DEVICE memory: db_host goes up, the column sums are
+** added to it row after row in float exactly as the caller's host loop would add them
+** (lang/ffn.c:301-305), the result comes back -- the host loop's bits, where the reference's
+** CUDA path keeps device accumulators that it flushes at the next sync (num/gpu_cuda.cu:
+** 3131-3193,9972-10030).  Synchronous.  -1 (the caller's host loop runs) for a host x: with this
+** backend's host GEMMs that is every call of the unchanged caller; a caller with a
+** device-resident backward and an arena adds straight into the gradient flat with
+** anni_colsum_add instead.
+*/
+int	gpu_mat_col_sum_add(ann_real *db_host, const ann_real *x, int rows, int cols);
+
 /* ---- the optimizer step ------------------------------------------------ */
 
 /* num/gpu.h:121 -- decoupled weight decay used by the next step (negative -> 0; sticky). */

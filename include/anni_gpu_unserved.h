@@ -82,7 +82,6 @@ int	gpu_ce_bias_fused(void);
 int	gpu_ce_bf16_delta_done(const ann_real *logits);
 int	gpu_ce_nll_rows(const ann_real *logits, const int *tgt, int rows, int V, float *out);
 int	gpu_posenc_add_packed(ann_real *x, int B, int T, int D);
-int	gpu_mat_col_sum_add(ann_real *db_host, const ann_real *x, int rows, int cols);
 int	gpu_relu_backward(ann_real *dx, const ann_real *x_pre_relu_or_mask, int n);
 int	gpu_ffn_relu_bwd_fused(mat *dh, const mat *hidden, ann_real *db1_host);
 int	gpu_act_bf16_only(const mat *m);

@@ -165,3 +165,33 @@ def test_argument_checks(gpu):
     assert gpu.anni_colsum_add(d.ptr, d.ptr, None, 4, (1 << 24) + 1) == -1
     assert gpu.anni_colsum_add(d.ptr, d.ptr, None, 0, 4) == 0
     d.free()
+
+
+def test_the_references_own_entry_point(gpu, oracle):
+    """gpu_mat_col_sum_add (num/gpu.h:195-199), the call of lang/ffn.c:298,355: a device matrix is
+    summed into the caller's HOST bias gradient with the host loop's bits, over several calls
+    (gradient accumulation: the vector is not zero at the second call); a host matrix is declined,
+    and the caller's own loop runs."""
+    import ctypes as C
+    from anni_amd.lm_adam import DeviceBuffer
+    gpu.gpu_mat_col_sum_add.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int]
+    gpu.gpu_mat_col_sum_add.restype = C.c_int
+    rng = np.random.default_rng(77)
+    for rows, cols in ((1, 1), (130, 257), (1000, 1536), (64, 6272)):
+        db = wide(rng, cols)
+        want = db.copy()
+        for _call in range(3):
+            x = wide(rng, (rows, cols))
+            d_x = DeviceBuffer(x.nbytes)
+            d_x.upload(x)
+            assert gpu.gpu_mat_col_sum_add(db.ctypes.data, d_x.ptr, rows, cols) == 0
+            oracle.colsum_add(want, x)
+            assert same_bits(db, want), (rows, cols, _call)
+            d_x.free()
+    x = wide(rng, (8, 16))
+    db = np.zeros(16, np.float32)
+    assert gpu.gpu_mat_col_sum_add(db.ctypes.data, x.ctypes.data, 8, 16) == -1      # host matrix
+    assert not db.any()
+    assert gpu.gpu_mat_col_sum_add(None, x.ctypes.data, 8, 16) == -1
+    assert gpu.gpu_mat_col_sum_add(db.ctypes.data, x.ctypes.data, 0, 16) == -1
+    assert gpu.gpu_debug_last_error() == b""             # declining is not an error
