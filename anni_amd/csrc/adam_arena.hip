@@ -409,6 +409,9 @@ static anni_adam *create_body(const anni_tensor *tensors, int n_tensors,
 			if (!ok) {
 				unplace(&pl);
 				pv->arena = nullptr;
+			} else if (z.n_slots > 0 && z.p_bytes >= kPlaceMin) {
+				pl.gbps = probe(opt);
+				pv->probe_gbps = pl.gbps;
 			}
 		}
 	}

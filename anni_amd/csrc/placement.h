@@ -32,10 +32,12 @@ constexpr size_t kPlaceMin = (size_t)256 << 20;
 ** requested one after the other with 16 GiB of ballast in between (the allocator works its way
 ** down through the sections), each timed against `ref`, until one is at least 7 % faster than the
 ** same launch inside a single block or memory runs low; the best one is kept, the others and
-** the ballast are returned.  Both probe areas -- the first 8 bytes per probe element of `ref`, the
-** first 18 of every candidate -- are zero-filled and left zero, so `ref` must not hold data
-** there.  *ratio (may be NULL) receives time(one block) / time(ref + result); 1.0 when nothing
-** was measured.  NULL when the allocation itself fails.  Synchronises the compute stream.
+** the ballast are returned.  Both probe areas -- the first 18 bytes per probe element of `ref` and of
+** every candidate -- are zero-filled and left zero, so `ref` must not hold data there.  *ratio
+** (may be NULL) receives time(one block) / time(ref + result), "one block" being the slower of
+** `ref` alone and the first candidate alone; 1.0 when nothing was measured.  A ratio near 1 with
+** a fast arena happens too: memory the driver reuses after frees is often pieced together from
+** several sections already, and then there is nothing left to gain.  NULL when the allocation itself fails.  Synchronises the compute stream.
 */
 void	*alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio);
 

@@ -103,10 +103,10 @@ void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio)
 
 	if (ratio)
 		*ratio = 1.0;
-	/* probe size: 8 bytes per element inside ref, 18 inside a candidate (for the one-block timing) */
+	/* probe size: 18 bytes per element inside ref and inside a candidate (for the one-block timings) */
 	n = kProbeElems;
-	if ((size_t)n * 8 > ref_bytes)
-		n = (int64_t)(ref_bytes / 8);
+	if ((size_t)n * 18 > ref_bytes)
+		n = (int64_t)(ref_bytes / 18);
 	if ((size_t)n * 18 > bytes)
 		n = (int64_t)(bytes / 18);
 	n = n / kTile * kTile;
@@ -122,7 +122,7 @@ void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio)
 	(void)free_bytes_now(&total);
 	const size_t margin = total / 20 > ((size_t)8 << 30) ? total / 20 : ((size_t)8 << 30);
 
-	if (launch_fill_bytes(st, ref, 0, (size_t)n * 8) != 0)
+	if (launch_fill_bytes(st, ref, 0, (size_t)n * 18) != 0)
 		return nullptr;
 	for (int it = 0; it < kMaxCandidates; it++) {
 		void *c = nullptr;
@@ -138,8 +138,17 @@ void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio)
 		if (launch_fill_bytes(st, c, 0, (size_t)n * 18) != 0)
 			break;
 		if (it == 0) {
-			t_same = probe_ms((char *)c + 10 * n, (char *)c, n);	/* all five flats in one block */
-			if (t_same <= 0.0)
+			/*
+			** All five flats in one block, timed inside `ref` and inside the first candidate:
+			** the slower of the two is the reference.  (A block that the driver pieced together
+			** from memory of several sections -- it does so when it reuses freed memory -- is
+			** fast by itself and would make every pair look no better than "one block".)
+			*/
+			const double t_ref = probe_ms((char *)ref + 10 * n, (char *)ref, n);
+			const double t_c = probe_ms((char *)c + 10 * n, (char *)c, n);
+
+			t_same = t_ref > t_c ? t_ref : t_c;
+			if (t_ref <= 0.0 || t_c <= 0.0)
 				break;
 		}
 		t_pair = probe_ms((char *)ref, (char *)c, n);

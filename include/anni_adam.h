@@ -135,8 +135,10 @@ int	anni_adam_is_split(const anni_adam *opt);
 /*
 ** What creation measured: time of the update with all flats in one block / time on this arena's
 ** two blocks, on a probe of 64 M elements (>= 1.07: the halves lie in different sections; ~1.0:
-** no such memory was found; 1.0 exactly: compact or not measured), and the GB/s of algorithmic
-** traffic the update then reached on the whole arena (0: not measured; needs a gradient slot).
+** no such memory was found, or the blocks the driver handed out are pieced together from several
+** sections already and there was nothing to gain; 1.0 exactly: compact or not measured), and the
+** GB/s of algorithmic traffic the update then reached on the whole arena, whatever its layout
+** (0: not measured; needs a gradient slot and a parameter flat of 256 MiB or more).
 */
 double	anni_adam_apart_ratio(const anni_adam *opt);
 double	anni_adam_probe_gbps(const anni_adam *opt);
