@@ -3,6 +3,8 @@
 ** on scratch flats (see placement.h).  No counterpart in the reference.
 */
 #include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 #include <vector>
 #include "adam_kernels.h"
@@ -13,9 +15,8 @@ namespace anni {
 
 static const int64_t kProbeElems = (int64_t)64 << 20;	/* 0.34 ms per launch; shorter launches tell less */
 static const int64_t kProbeMinElems = (int64_t)8 << 20;
-static const size_t kBallastStep = (size_t)16 << 30;
-static const size_t kBallastMax = (size_t)112 << 30;	/* a section is 96 GiB: enough to leave any of them */
-static const int kMaxCandidates = 24;
+static const size_t kProbeEvery = (size_t)8 << 30;	/* a block is timed about every 8 GiB of blocks */
+static const size_t kWalkMax = (size_t)200 << 30;	/* a section is 96 GiB: two of them, and some for gaps */
 static const double kApartRatio = 1.07;			/* measured 1.13 - 1.17 across a section boundary */
 
 /*
@@ -75,6 +76,19 @@ static double probe_ms(char *a0, char *b0, int64_t n)
 	return (double)ms / reps;
 }
 
+/* ANNI_PLACE_LOG=1: one line per candidate on stderr. */
+static bool place_log(void)
+{
+	static int on = -1;
+
+	if (on < 0) {
+		const char *e = getenv("ANNI_PLACE_LOG");
+
+		on = (e && e[0] == '1') ? 1 : 0;
+	}
+	return on == 1;
+}
+
 static size_t free_bytes_now(size_t *total)
 {
 	size_t fr = 0, tt = 0;
@@ -92,9 +106,8 @@ static size_t free_bytes_now(size_t *total)
 void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio)
 {
 	hipStream_t st = compute_stream();
-	std::vector<void *> ballast;
-	std::vector<void *> cands;
-	size_t ballast_bytes = 0;
+	std::vector<void *> blocks;
+	size_t walked = 0;
 	size_t total = 0;
 	double t_same = 0.0;
 	double best_ratio = 0.0;
@@ -121,10 +134,20 @@ void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio)
 	}
 	(void)free_bytes_now(&total);
 	const size_t margin = total / 20 > ((size_t)8 << 30) ? total / 20 : ((size_t)8 << 30);
+	/*
+	** The walk: blocks of `bytes` are requested one after the other and kept, so the allocator
+	** works its way down through device memory; about every 8 GiB one of them is timed.  The
+	** blocks in between are ballast of the SAME size as the candidates on purpose: requests of
+	** one size fill the gaps the allocator has in the order it would fill them for the
+	** candidates too, whereas large aligned ballast leaves gaps near the top in which small
+	** candidates then all end up (seen with 1.5 GiB candidates and 16 GiB ballast: eight
+	** candidates, 112 GiB walked, none of them out of the first section).
+	*/
+	const size_t every = bytes >= kProbeEvery ? 1 : (kProbeEvery + bytes - 1) / bytes;
 
 	if (launch_fill_bytes(st, ref, 0, (size_t)n * 18) != 0)
 		return nullptr;
-	for (int it = 0; it < kMaxCandidates; it++) {
+	for (size_t it = 0; walked < kWalkMax; it++) {
 		void *c = nullptr;
 		double t_pair;
 
@@ -134,7 +157,10 @@ void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio)
 			(void)hipGetLastError();
 			break;
 		}
-		cands.push_back(c);
+		blocks.push_back(c);
+		walked += bytes;
+		if (it % every != 0)
+			continue;
 		if (launch_fill_bytes(st, c, 0, (size_t)n * 18) != 0)
 			break;
 		if (it == 0) {
@@ -154,39 +180,30 @@ void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio)
 		t_pair = probe_ms((char *)ref, (char *)c, n);
 		if (t_pair <= 0.0)
 			break;
+		if (place_log())
+			fprintf(stderr, "[place] block %zu at %p (%.2f GiB): one block %.4f ms, with ref %p %.4f ms, "
+			    "ratio %.3f, walked %.0f GiB, free %.1f GiB\n", it, c, (double)bytes / 1073741824.0,
+			    t_same, ref, t_pair, t_same / t_pair, (double)walked / 1073741824.0,
+			    (double)free_bytes_now(nullptr) / 1073741824.0);
 		if (best < 0 || t_same / t_pair > best_ratio) {
-			best = it;
+			best = (int)it;
 			best_ratio = t_same / t_pair;
 		}
 		if (best_ratio >= kApartRatio)
 			break;
-		if (ballast_bytes + kBallastStep > kBallastMax)
-			break;
-		if (free_bytes_now(nullptr) >= kBallastStep + bytes + margin) {
-			void *b = nullptr;
-
-			if (hipMalloc(&b, kBallastStep) == hipSuccess) {
-				ballast.push_back(b);
-				ballast_bytes += kBallastStep;
-			} else {
-				(void)hipGetLastError();
-			}
-		}
 	}
 	(void)hipStreamSynchronize(st);
-	if (best < 0 && !cands.empty())
+	if (best < 0 && !blocks.empty())
 		best = 0;
-	for (size_t i = 0; i < cands.size(); i++)
+	for (size_t i = 0; i < blocks.size(); i++)
 		if ((int)i != best)
-			(void)hipFree(cands[i]);
-	for (void *b : ballast)
-		(void)hipFree(b);
+			(void)hipFree(blocks[i]);
 	(void)hipGetLastError();
 	if (best < 0)
 		return nullptr;
 	if (ratio && best_ratio > 0.0)
 		*ratio = best_ratio;
-	return cands[(size_t)best];
+	return blocks[(size_t)best];
 }
 
 } /* namespace anni */
