@@ -43,9 +43,10 @@ extern "C" {
 ** than when one holds them all.  SPLIT makes two allocations of exactly the size of their
 ** contents -- p, m and the tables in one; v, the twins and the gradient slots in the other -- and
 ** looks for the second in another section by timing the update on the (still empty) flats:
-** candidates are requested with ballast in between until one is fast or memory runs low, and
-** everything but the arena is returned before anni_adam_create returns (for a moment up to
-** ~120 GiB more than the arena are held; with little memory free the search just ends sooner).
+** blocks of its size are requested one after the other and kept, every 8 GiB one is timed, until
+** one is fast, 200 GiB have been walked or memory runs low, and everything but the arena is
+** returned before anni_adam_create returns (for a moment up to ~200 GiB more than the arena are
+** held; with little memory free the search just ends sooner).
 ** COMPACT is one allocation.  AUTO splits when the parameter flat has 256 MiB or more.
 */
 #define ANNI_LAYOUT_AUTO	0
