@@ -610,8 +610,12 @@ static void *pool_take(size_t nbytes)
 	return chunk_take(g_chunks.back(), need);
 }
 
-/* g_pool_mu held.  True when p was a block of a pool (now free again). */
-static bool pool_give(void *p)
+/*
+** g_pool_mu held.  1 when p was a block of a pool (now free again), 0 when p lies in no chunk,
+** -1 when it points into a chunk without being the start of a live block (a caller's mistake:
+** nothing is freed).
+*/
+static int pool_give(void *p)
 {
 	for (PoolChunk &c : g_chunks) {
 		if ((char *)p < c.base || (char *)p >= c.base + c.bytes)
@@ -632,11 +636,11 @@ static bool pool_give(void *p)
 				c.blocks[i - 1].bytes += c.blocks[i].bytes;
 				c.blocks.erase(c.blocks.begin() + (long)i);
 			}
-			return true;
+			return 1;
 		}
-		return false;		/* inside a chunk, but not the start of a live block */
+		return -1;
 	}
-	return false;
+	return 0;
 }
 
 /* g_pool_mu held.  Bytes of chunks that are reserved but hold no block. */
@@ -722,10 +726,19 @@ void gpu_free(void *p)
 		}
 	}
 	{
-		std::lock_guard<std::mutex> lk(g_pool_mu);
+		int given;
 
-		if (pool_give(p))
+		{
+			std::lock_guard<std::mutex> lk(g_pool_mu);
+
+			given = pool_give(p);
+		}
+		if (given > 0)
 			return;
+		if (given < 0) {
+			(void)hip_ok(hipErrorInvalidDevicePointer, "gpu_free: not the start of a block");
+			return;
+		}
 	}
 	(void)hip_ok(hipFree(p), "hipFree");
 }

@@ -452,6 +452,9 @@ def test_large_allocations_are_dealt_to_two_pools(gpu):
     assert all(p % (2 << 20) == 0 for p in ptrs)
     small = gpu.gpu_malloc(1 << 20)                      # small blocks are ordinary allocations
     assert small and pool_of(small) is None
+    gpu.gpu_debug_last_error()
+    gpu.gpu_free(ptrs[1] + 4096)                         # not the start of a block: refused, nothing freed
+    assert b"not the start of a block" in gpu.gpu_debug_last_error()
     gpu.gpu_free(ptrs[1])
     again = gpu.gpu_malloc(4 * n)                        # a freed block is reused (first fit)
     assert again == ptrs[1]
