@@ -16,6 +16,7 @@
 #include "anni_gpu.h"
 #include "backend_state.h"
 #include "placement.h"
+#include "pool_chunks.h"
 
 namespace anni {
 
@@ -501,18 +502,6 @@ void gpu_op_prof_dump(void)
 ** being created, gives them back first; gpu_mem_info counts them as free.
 ** ANNI_MALLOC_PLACE=0 switches all of this off (every block a plain hipMalloc).
 */
-struct PoolBlock {
-	size_t	off;
-	size_t	bytes;
-	bool	used;
-};
-struct PoolChunk {
-	char			*base;
-	size_t			bytes;
-	int			pool;
-	size_t			live;		/* bytes handed out */
-	std::vector<PoolBlock>	blocks;		/* sorted by offset, covering the chunk */
-};
 static std::vector<PoolChunk> g_chunks;
 static size_t g_pool_live[2];
 
@@ -531,21 +520,12 @@ static bool place_on(void)
 /* First fit inside one chunk.  g_pool_mu held. */
 static void *chunk_take(PoolChunk &c, size_t need)
 {
-	for (size_t i = 0; i < c.blocks.size(); i++) {
-		if (c.blocks[i].used || c.blocks[i].bytes < need)
-			continue;
-		if (c.blocks[i].bytes > need) {
-			const PoolBlock rest = { c.blocks[i].off + need, c.blocks[i].bytes - need, false };
+	const size_t off = c.take(need);
 
-			c.blocks[i].bytes = need;
-			c.blocks.insert(c.blocks.begin() + (long)i + 1, rest);
-		}
-		c.blocks[i].used = true;
-		c.live += need;
-		g_pool_live[c.pool] += need;
-		return c.base + c.blocks[i].off;
-	}
-	return nullptr;
+	if (off == (size_t)-1)
+		return nullptr;
+	g_pool_live[c.pool] += need;
+	return c.base + off;
 }
 
 /* The largest free block of the chunks of `pool`: scratch for the placement probe.  g_pool_mu held. */
@@ -555,13 +535,13 @@ static char *pool_scratch(int pool, size_t *bytes)
 
 	*bytes = 0;
 	for (PoolChunk &c : g_chunks) {
-		if (c.pool != pool)
-			continue;
-		for (const PoolBlock &b : c.blocks)
-			if (!b.used && b.bytes > *bytes) {
-				*bytes = b.bytes;
-				best = c.base + b.off;
-			}
+		size_t n = 0;
+		const size_t off = c.largest_free(&n);
+
+		if (c.pool == pool && n > *bytes) {
+			*bytes = n;
+			best = c.base + off;
+		}
 	}
 	return best;
 }
@@ -575,7 +555,6 @@ static void *pool_take(size_t nbytes)
 	size_t chunk_bytes = 4 * need;
 	char *scratch;
 	void *mem = nullptr;
-	PoolChunk c;
 
 	for (PoolChunk &have : g_chunks)
 		if (have.pool == pool) {
@@ -601,12 +580,7 @@ static void *pool_take(size_t nbytes)
 	}
 	if (!mem)
 		return nullptr;
-	c.base = (char *)mem;
-	c.bytes = chunk_bytes;
-	c.pool = pool;
-	c.live = 0;
-	c.blocks.push_back(PoolBlock{ 0, chunk_bytes, false });
-	g_chunks.push_back(c);
+	g_chunks.push_back(PoolChunk((char *)mem, chunk_bytes, pool));
 	return chunk_take(g_chunks.back(), need);
 }
 
@@ -620,25 +594,12 @@ static int pool_give(void *p)
 	for (PoolChunk &c : g_chunks) {
 		if ((char *)p < c.base || (char *)p >= c.base + c.bytes)
 			continue;
-		const size_t off = (size_t)((char *)p - c.base);
+		const size_t n = c.give((size_t)((char *)p - c.base));
 
-		for (size_t i = 0; i < c.blocks.size(); i++) {
-			if (c.blocks[i].off != off || !c.blocks[i].used)
-				continue;
-			c.blocks[i].used = false;
-			c.live -= c.blocks[i].bytes;
-			g_pool_live[c.pool] -= c.blocks[i].bytes;
-			if (i + 1 < c.blocks.size() && !c.blocks[i + 1].used) {
-				c.blocks[i].bytes += c.blocks[i + 1].bytes;
-				c.blocks.erase(c.blocks.begin() + (long)i + 1);
-			}
-			if (i > 0 && !c.blocks[i - 1].used) {
-				c.blocks[i - 1].bytes += c.blocks[i].bytes;
-				c.blocks.erase(c.blocks.begin() + (long)i);
-			}
-			return 1;
-		}
-		return -1;
+		if (n == 0)
+			return -1;
+		g_pool_live[c.pool] -= n;
+		return 1;
 	}
 	return 0;
 }

@@ -157,3 +157,18 @@ def test_c99_caller_with_the_reference_flags(tmp_path):
     assert lr[0] == 0.01 and lr[1] == 1.0 and abs(lr[2] - 0.5) < 1e-15 and abs(lr[3]) < 1e-15
     assert out[1].startswith("backend hip-gfx950 available ")
     assert out[2].startswith("create declined") or out[2].startswith("create ok n 4160 t 1 norm 0")
+
+
+def test_pool_chunk_bookkeeping_on_the_host(tmp_path):
+    """The first-fit block bookkeeping of gpu_malloc's pools (anni_amd/csrc/pool_chunks.h) has no
+    device call in it: a random sequence of 20000 takes and gives against a byte map."""
+    import shutil
+    import subprocess
+    if not shutil.which("g++"):
+        pytest.skip("no g++")
+    exe = str(tmp_path / "pool_chunks_test")
+    subprocess.check_call(["g++", "-std=c++17", "-O2", "-Wall", "-Wextra", "-Werror",
+                           "-I", os.path.join(ROOT, "anni_amd", "csrc"),
+                           os.path.join(ROOT, "tests", "c", "pool_chunks_test.cpp"), "-o", exe])
+    out = subprocess.check_output([exe], timeout=120).decode()
+    assert out.startswith("ok takes "), out
