@@ -1258,6 +1258,7 @@ static int g_warmup_steps;
 static int g_decay_steps;
 static int g_decay_kind;	/* 0 none, 1 linear, 2 cosine (any other name: cosine, as the reference) */
 static int g_sched_from;
+static double g_lr_override;	/* the lr field of the reference's train_control (lm_train.c:104-105); <= 0: none */
 
 void anni_lr_set_schedule(int warmup_steps, int decay_steps, const char *kind)
 {
@@ -1276,11 +1277,18 @@ void anni_lr_set_sched_from(int from)
 	g_sched_from = from < 0 ? 0 : from;
 }
 
+void anni_lr_set_override(double lr)
+{
+	g_lr_override = lr;
+}
+
 double anni_lr_step(double base_lr, int step)
 {
 	double q;
 	int u;
 
+	if (g_lr_override > 0.0)
+		return g_lr_override;		/* lm_train.c:104-105 */
 	step -= g_sched_from;
 	if (step < 0)
 		step = 0;

@@ -121,6 +121,7 @@ _PROTOS = {
     "anni_gpu_reload_switches": (None, []),
     "anni_lr_set_schedule": (None, [C.c_int, C.c_int, C.c_char_p]),
     "anni_lr_set_sched_from": (None, [C.c_int]),
+    "anni_lr_set_override": (None, [C.c_double]),
     "anni_lr_step": (C.c_double, [C.c_double, C.c_int]),
     "anni_gpu_stream": (C.c_void_p, []),
     "anni_gpu_set_stream": (None, [C.c_void_p]),

@@ -221,6 +221,12 @@ int	anni_adam_read_state(anni_adam *opt, int fd, int *epoch, int *step);
 /* lm_train_step_lr and its setters (lang/lm_train.c:98-124,398-411); kind "none" / "linear" / "cosine". */
 void	anni_lr_set_schedule(int warmup_steps, int decay_steps, const char *kind);
 void	anni_lr_set_sched_from(int from);
+/*
+** The live control of the reference's training loop (train_control.lr set through
+** lm_train_set_control, lang/train_progress.h:46-56, lm_train.c:93-105): a value > 0 is returned
+** by anni_lr_step whatever the schedule says; <= 0 gives the schedule back.
+*/
+void	anni_lr_set_override(double lr);
 double	anni_lr_step(double base_lr, int step);
 
 /* ---- stream plumbing ---------------------------------------------------- */

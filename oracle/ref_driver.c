@@ -14,6 +14,7 @@
 #include "lm_adam.h"
 #include "lm_serialize.h"
 #include "lm_train.h"
+#include "train_progress.h"
 #include "layernorm.h"
 #include "lm_bench.h"
 
@@ -332,6 +333,21 @@ double ref_step_lr(double base_lr, int step, int warmup, int decay_steps,
 	lr = lm_train_step_lr(base_lr, step);
 	lm_train_set_lr_sched_from(0);
 	lm_train_set_lr_schedule(0, 0, "none");
+	return lr;
+}
+
+/* lm_train_step_lr under a live control whose lr field is `ctl_lr` (lang/train_progress.h:46-56). */
+double ref_step_lr_controlled(double base_lr, int step, int warmup, int decay_steps,
+	const char *kind, double ctl_lr)
+{
+	train_control ctl;
+	double lr;
+
+	memset(&ctl, 0, sizeof(ctl));
+	ctl.lr = ctl_lr;
+	lm_train_set_control(&ctl);
+	lr = ref_step_lr(base_lr, step, warmup, decay_steps, kind, 0);
+	lm_train_set_control(NULL);
 	return lr;
 }
 

@@ -120,6 +120,21 @@ def test_lr_schedule_host_logic(oracle):
             assert got == want == oracle.lr(3e-4, int(s), int(w), int(d), k, int(frm))
     # setters clamp negatives (lm_train.c:398-411)
     assert f(1.0, 5, -3, -7, "cosine", -2) == 1.0
+    # the live control (train_control.lr, lm_train.c:104-105): > 0 wins over any schedule, <= 0 does not
+    from anni_amd import lib
+    L = lib.load()
+    for ctl in (2.5e-5, 0.0, -1.0):
+        L.anni_lr_set_override(ctl)
+        for s in (0, 50, 600, 5000):
+            got = f(3e-4, s, 100, 1000, "cosine", 0)
+            want = ctl if ctl > 0 else oracle.lr(3e-4, s, 100, 1000, "cosine", 0)
+            assert got == want
+            if oracle.ref_available():
+                R = oracle.ref()
+                R.ref_step_lr_controlled.argtypes = [C.c_double, C.c_int, C.c_int, C.c_int, C.c_char_p, C.c_double]
+                R.ref_step_lr_controlled.restype = C.c_double
+                assert R.ref_step_lr_controlled(3e-4, s, 100, 1000, b"cosine", ctl) == got
+    L.anni_lr_set_override(0.0)
 
 
 def test_layout_parameter_counts():
