@@ -40,6 +40,7 @@ struct anni_adam_priv {
 	char			*grad_slots;	/* the arena's gradient flats (NULL when external) */
 	size_t			grad_slot_bytes;	/* distance between consecutive slots */
 	int			n_grad_slots;
+	int			logged_t;	/* the step whose messages anni_adam_sync_stats has printed */
 	int			split;		/* 1: two allocations (see the layout note in anni_adam_create) */
 	double			probe_gbps;	/* update throughput measured at creation (0: not measured) */
 	std::vector<int64_t>	offsets;
@@ -913,6 +914,28 @@ int anni_adam_sync_stats(anni_adam *opt)
 	opt->last_grad_scale = pv->h_state->grad_scale;
 	opt->last_skipped = pv->h_state->skipped;
 	opt->last_clipped = pv->h_state->clipped;
+	/*
+	** The reference's messages for the step just read back (lm_adam.c:479-487), once per step:
+	** a skipped step always, the norm every ANN_GNORM_EVERY steps.  The step itself never waits
+	** for the host, so they appear when the caller asks for the numbers.
+	*/
+	if (pv->logged_t != opt->t && (opt->grad_clip > 0.0 || opt->cfg.skip_nonfinite)) {
+		static int every = -1;
+
+		if (every < 0) {
+			const char *e = getenv("ANN_GNORM_EVERY");
+
+			every = e ? atoi(e) : 0;
+			if (every < 0)
+				every = 0;
+		}
+		pv->logged_t = opt->t;
+		if (opt->last_skipped)
+			fprintf(stderr, "[adam] step %d skipped: grad norm %g\n", opt->t, opt->last_grad_norm);
+		else if (every > 0 && opt->t % every == 0)
+			fprintf(stderr, "[adam] step %d grad norm %.4g%s\n", opt->t, opt->last_grad_norm,
+			    opt->last_clipped ? " (clipped)" : "");
+	}
 	return 0;
 }
 

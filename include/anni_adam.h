@@ -202,7 +202,12 @@ int	anni_adam_quantize_grads_static(anni_adam *opt, const float *d_src);
 int	anni_adam_step_scaled(anni_adam *opt, double lr, double grad_scale);
 /* lm_adam_step. */
 int	anni_adam_step(anni_adam *opt, double lr);
-/* Waits for the stream and fills last_sumsq / last_grad_norm / last_grad_scale / last_skipped / last_clipped. */
+/*
+** Waits for the stream and fills last_sumsq / last_grad_norm / last_grad_scale / last_skipped /
+** last_clipped; prints the reference's messages for that step on stderr (lm_adam.c:479-487):
+** "[adam] step T skipped: grad norm G" for a skipped step, and with ANN_GNORM_EVERY=N
+** "[adam] step T grad norm G (clipped)" every N steps.
+*/
 int	anni_adam_sync_stats(anni_adam *opt);
 
 /*

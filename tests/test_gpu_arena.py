@@ -174,7 +174,7 @@ def test_lr_nonpositive_is_a_noop(gpu):
 
 
 @pytest.mark.parametrize("bad,where", [(np.nan, 0), (np.inf, 5000 + 3 + 17), (-np.inf, -1)])
-def test_nonfinite_skip_leaves_state_bit_identical(gpu, oracle, bad, where):
+def test_nonfinite_skip_leaves_state_bit_identical(gpu, oracle, bad, where, capfd):
     rng = np.random.default_rng(31)
     opt = make(gpu, RAGGED, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True)
     n = opt.n
@@ -202,6 +202,12 @@ def test_nonfinite_skip_leaves_state_bit_identical(gpu, oracle, bad, where):
                 assert same_bits(a, b) if a.dtype == np.float32 else (a == b).all()
         assert same_bits(after[0], P) and same_bits(after[1], M) and same_bits(after[2], V)
         assert not opt.download("grad").any()
+        opt.sync_stats()                                 # a second read of the same step prints nothing more
+    # the reference's message for the skipped step (lm_adam.c:479-480), once
+    err = capfd.readouterr().err
+    lines = [ln for ln in err.splitlines() if ln.startswith("[adam] step ")]
+    assert len(lines) == 1 and lines[0].startswith("[adam] step 3 skipped: grad norm "), err
+    assert lines[0].split()[-1] in ("nan", "-nan", "inf")
     opt.free()
 
 
