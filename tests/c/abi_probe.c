@@ -8,6 +8,7 @@
 #include "anni_gpu.h"
 #include "anni_gpu_unserved.h"
 #include "anni_adam.h"
+#include "anni_bench.h"
 
 int main(void)
 {
