@@ -1,6 +1,6 @@
 /*
 ** A C99 caller of the library, compiled with the reference's own flags (Makefile:21:
-** -W -Wall -ansi -pedantic -std=c99): the three headers are plain C, the symbols link, and the
+** -W -Wall -ansi -pedantic -std=c99): the four headers are plain C, the symbols link, and the
 ** host-only entry points answer.  Prints the learning rate at a few schedule steps, which the
 ** reference's test pins (tests/test_ann.c:866-879), and what the backend says about itself.
 */
