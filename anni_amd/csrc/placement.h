@@ -31,8 +31,8 @@ constexpr size_t kPlaceMin = (size_t)256 << 20;
 ** [ref, ref + ref_bytes): memory of another section when one can be had.  Blocks of `bytes` are
 ** requested one after the other and kept (the allocator works its way down through the
 ** sections), about every 8 GiB one of them is timed against `ref`, until one is at least 7 %
-** faster than the same launch inside a single block, 200 GiB have been walked or memory runs
-** low; the best one is kept, all others are returned.  Both probe areas -- the first 18 bytes per probe element of `ref` and of
+** faster than the same launch inside a single block, 200 GiB have been walked (ANNI_PLACE_MAX_GIB
+** sets another limit) or memory runs low; the best one is kept, all others are returned.  Both probe areas -- the first 18 bytes per probe element of `ref` and of
 ** every candidate -- are zero-filled and left zero, so `ref` must not hold data there.  *ratio
 ** (may be NULL) receives time(one block) / time(ref + result), "one block" being the slower of
 ** `ref` alone and the first candidate alone; 1.0 when nothing was measured.  A ratio near 1 with

@@ -89,6 +89,21 @@ static bool place_log(void)
 	return on == 1;
 }
 
+/* How far the walk may go: ANNI_PLACE_MAX_GIB (default 200; 0 = no walk, the first block is taken). */
+static size_t walk_max(void)
+{
+	static long gib = -1;
+
+	if (gib < 0) {
+		const char *e = getenv("ANNI_PLACE_MAX_GIB");
+
+		gib = e && *e ? atol(e) : (long)(kWalkMax >> 30);
+		if (gib < 0 || gib > 1024)
+			gib = (long)(kWalkMax >> 30);
+	}
+	return (size_t)gib << 30;
+}
+
 static size_t free_bytes_now(size_t *total)
 {
 	size_t fr = 0, tt = 0;
@@ -147,7 +162,7 @@ void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio)
 
 	if (launch_fill_bytes(st, ref, 0, (size_t)n * 18) != 0)
 		return nullptr;
-	for (size_t it = 0; walked < kWalkMax; it++) {
+	for (size_t it = 0; it == 0 || walked < walk_max(); it++) {
 		void *c = nullptr;
 		double t_pair;
 
