@@ -16,8 +16,8 @@
 #include <vector>
 #include "adam_kernels.h"
 #include "anni_adam.h"
-#include "anni_bench.h"
 #include "anni_gpu.h"
+#include "anni_hooks.h"
 #include "backend_state.h"
 #include "placement.h"
 
@@ -25,6 +25,28 @@ using namespace anni;
 
 /* Step state (128 bytes) + the ticket counters of the norm's second stage. */
 static const size_t kStateBytes = 128 + ((kTicketBytes + 255) / 256) * 256;
+
+static size_t elem_bytes(int type)
+{
+	return type == ANNI_F32 ? 4 : type == ANNI_BF16 ? 2 : 1;
+}
+
+static size_t round_up(size_t x, size_t a)
+{
+	return (x + a - 1) / a * a;
+}
+
+/* Byte sizes of the flats of one arena. */
+struct Sizes {
+	int64_t	n;
+	int	n_tensors;
+	int64_t	n_tiles;
+	int	n_slots;
+	size_t	p_bytes;
+	size_t	mv_bytes;
+	size_t	tw_bytes;
+	size_t	g_bytes;	/* one gradient slot, rounded up to 2 MiB */
+};
 
 struct anni_adam_priv {
 	void			*arena;		/* p, m and the tables (split), or everything (compact) */
@@ -53,31 +75,14 @@ struct anni_adam_priv {
 	PackDesc		*d_packs;
 	float			*d_tile_amax;	/* per-wavefront max |p| of every whole tile */
 	int			fp8_twins;	/* 1: some tensor keeps an E4M3 twin */
-	float			der_ms;		/* E4M3 pass time summed by anni_adam_time_steps */
 	/* scratch of anni_adam_quantize_grads, allocated at its first call: per-tensor max words, then the tile maxima */
 	void			*gq_scratch;
-};
-
-static size_t elem_bytes(int type)
-{
-	return type == ANNI_F32 ? 4 : type == ANNI_BF16 ? 2 : 1;
-}
-
-static size_t round_up(size_t x, size_t a)
-{
-	return (x + a - 1) / a * a;
-}
-
-/* Byte sizes of the flats of one arena. */
-struct Sizes {
-	int64_t	n;
-	int	n_tensors;
-	int64_t	n_tiles;
-	int	n_slots;
-	size_t	p_bytes;
-	size_t	mv_bytes;
-	size_t	tw_bytes;
-	size_t	g_bytes;	/* one gradient slot, rounded up to 2 MiB */
+	/* anni_adam_set_offload */
+	Sizes			z;		/* what the arena was laid out for */
+	int			mv_apart;	/* 1: m and v are blocks of their own (gpu_malloc), not parts of the arena's */
+	int			offload;	/* 1: m and v leave the device after every step */
+	void			*h_m;		/* page-locked homes of m and v while they are away */
+	void			*h_v;
 };
 
 /* One or two device allocations with the flats laid out in them. */
@@ -361,6 +366,7 @@ static anni_adam *create_body(const anni_tensor *tensors, int n_tensors,
 	z.mv_bytes = (size_t)n * elem_bytes(cfg->moment_type);
 	z.tw_bytes = cfg->twins ? (size_t)n * 2 : 0;
 	z.g_bytes = round_up((size_t)n * elem_bytes(cfg->grad_type), big);
+	pv->z = z;
 	tile_seg.resize((size_t)z.n_tiles);
 	{
 		int s = 0;
@@ -451,6 +457,14 @@ void anni_adam_free(anni_adam **popt)
 	if (opt->priv) {
 		if (device_ready())
 			(void)hipStreamSynchronize(compute_stream());
+		if (opt->priv->mv_apart) {
+			gpu_free(opt->d_m);
+			gpu_free(opt->d_v);
+		}
+		if (opt->priv->h_m)
+			(void)hip_ok(hipHostFree(opt->priv->h_m), "offload hipHostFree");
+		if (opt->priv->h_v)
+			(void)hip_ok(hipHostFree(opt->priv->h_v), "offload hipHostFree");
 		if (opt->priv->arena)
 			(void)hip_ok(hipFree(opt->priv->arena), "arena hipFree");
 		if (opt->priv->arena2)
@@ -644,11 +658,6 @@ int anni_adam_enable_derived(anni_adam *opt, const anni_pack *packs, int n_packs
 	}
 }
 
-float anni_adam_timed_derived_ms(const anni_adam *opt)
-{
-	return opt && opt->priv ? opt->priv->der_ms : 0.0f;
-}
-
 int anni_adam_zero_grad(anni_adam *opt)
 {
 	if (!opt || !opt->d_grad)
@@ -803,6 +812,210 @@ static unsigned int *ticket_word(const anni_adam_priv *pv)
 ** One step; ev (may be NULL) = four events recorded before the step, after the sum of squares, after
 ** the update and after the derived outputs; an entry that is NULL is not recorded.
 */
+/* ---- m and v off the device between steps (lm_adam.c:211-214,295-334) ----------------------- */
+
+/*
+** The reference can park the moments on the host between steps (lm_adam_set_offload): after a
+** step adam_offload_mv reads d_m and d_v back and frees them, the next step allocates and uploads
+** them again -- two of the five flats leave the device while forward and backward need the room.
+** Here m and v normally are parts of the arena's two blocks, which cannot be freed piecemeal, so
+** the first anni_adam_set_offload(opt, 1) re-houses the arena: m and v move into blocks of
+** their own (gpu_malloc: its pools keep the emptied chunks, so taking the blocks again costs
+** nothing and gpu_mem_info reads the same before and after every step), everything else into
+** two new blocks without room for them.  While the moments are away opt->d_m and opt->d_v are
+** NULL; their homes are two page-locked host buffers, raw copies of the stored type.
+*/
+static int mv_bring(anni_adam *opt)
+{
+	anni_adam_priv *pv = opt->priv;
+	hipStream_t st;
+
+	if (opt->d_m && opt->d_v)
+		return 0;
+	if (!pv->mv_apart || !pv->h_m || !pv->h_v)
+		return -1;
+	opt->d_m = gpu_malloc(pv->z.mv_bytes);
+	opt->d_v = gpu_malloc(pv->z.mv_bytes);
+	if (!opt->d_m || !opt->d_v) {
+		gpu_free(opt->d_m);
+		gpu_free(opt->d_v);
+		opt->d_m = opt->d_v = nullptr;
+		return -1;
+	}
+	st = compute_stream();
+	if (!hip_ok(hipMemcpyAsync(opt->d_m, pv->h_m, pv->z.mv_bytes, hipMemcpyHostToDevice, st), "offload h2d")
+	    || !hip_ok(hipMemcpyAsync(opt->d_v, pv->h_v, pv->z.mv_bytes, hipMemcpyHostToDevice, st), "offload h2d"))
+		return -1;
+	return 0;
+}
+
+static int mv_send(anni_adam *opt)
+{
+	anni_adam_priv *pv = opt->priv;
+	hipStream_t st;
+
+	if (!opt->d_m || !opt->d_v)
+		return 0;
+	if (!pv->mv_apart || !pv->h_m || !pv->h_v)
+		return -1;
+	st = compute_stream();
+	if (!hip_ok(hipMemcpyAsync(pv->h_m, opt->d_m, pv->z.mv_bytes, hipMemcpyDeviceToHost, st), "offload d2h")
+	    || !hip_ok(hipMemcpyAsync(pv->h_v, opt->d_v, pv->z.mv_bytes, hipMemcpyDeviceToHost, st), "offload d2h")
+	    || !hip_ok(sync_stream_and_deliver(), "offload sync"))
+		return -1;
+	gpu_free(opt->d_m);
+	gpu_free(opt->d_v);
+	opt->d_m = opt->d_v = nullptr;
+	return 0;
+}
+
+/* Runs `work` with the moments on the device: offloaded ones are brought back for it and sent away again. */
+template <typename F>
+static int with_moments(anni_adam *opt, F work)
+{
+	int rc;
+
+	if (mv_bring(opt) != 0)
+		return -1;
+	rc = work();
+	if (opt->priv->offload && mv_send(opt) != 0)
+		rc = -1;
+	return rc;
+}
+
+/* Moves m and v into blocks of their own and everything else into two new blocks without them. */
+static int rehouse_without_mv(anni_adam *opt)
+{
+	anni_adam_priv *pv = opt->priv;
+	hipStream_t st = compute_stream();
+	Sizes z = pv->z;
+	Placement pl;
+	void *m2, *v2;
+	char *old_a = (char *)pv->arena;
+	char *old_b = (char *)pv->arena2;
+	const float *old_gscale = (const float *)((char *)pv->d_segs
+	    - round_up((size_t)z.n_tensors * sizeof(float), 256));
+	const bool own_gscale = opt->d_gscale == old_gscale;
+	const size_t slots_bytes = (size_t)z.n_slots * z.g_bytes;
+	const size_t tables = tables_bytes(z);
+	long bound_slot = -1;
+	bool ok;
+
+	if (!hip_ok(sync_stream_and_deliver(), "offload sync"))
+		return -1;
+	if (pv->grad_slots && (char *)opt->d_grad >= pv->grad_slots
+	    && (char *)opt->d_grad < pv->grad_slots + slots_bytes)
+		bound_slot = (long)(((char *)opt->d_grad - pv->grad_slots) / (long)pv->grad_slot_bytes);
+	m2 = gpu_malloc(z.mv_bytes);
+	v2 = gpu_malloc(z.mv_bytes);
+	z.mv_bytes = 0;			/* the new blocks have no room for the moments */
+	if (!m2 || !v2 || !place(z, pv->split != 0, &pl)) {
+		gpu_free(m2);
+		gpu_free(v2);
+		return -1;
+	}
+	{
+		char *second = pl.b ? pl.b : pl.a;
+		char *old_second = old_b ? old_b : old_a;
+
+		ok = hip_ok(hipMemcpyAsync(m2, opt->d_m, pv->z.mv_bytes, hipMemcpyDeviceToDevice, st), "rehouse")
+		    && hip_ok(hipMemcpyAsync(v2, opt->d_v, pv->z.mv_bytes, hipMemcpyDeviceToDevice, st), "rehouse")
+		    && hip_ok(hipMemcpyAsync(pl.a + pl.off_p, opt->d_param, z.p_bytes, hipMemcpyDeviceToDevice, st), "rehouse")
+		    /* the tables, the partials and the step state lie in one run behind the per-tensor scales */
+		    && hip_ok(hipMemcpyAsync(pl.a + pl.off_gscale, old_gscale, tables, hipMemcpyDeviceToDevice, st), "rehouse")
+		    && (!z.tw_bytes || hip_ok(hipMemcpyAsync(second + pl.off_twin, opt->d_param_bf16, z.tw_bytes,
+		    hipMemcpyDeviceToDevice, st), "rehouse"))
+		    && (!slots_bytes || hip_ok(hipMemcpyAsync(second + pl.off_g, pv->grad_slots, slots_bytes,
+		    hipMemcpyDeviceToDevice, st), "rehouse"))
+		    && hip_ok(hipStreamSynchronize(st), "rehouse sync");
+		(void)old_second;
+	}
+	if (!ok) {
+		unplace(&pl);
+		gpu_free(m2);
+		gpu_free(v2);
+		return -1;
+	}
+	{
+		void *ext_grad = bound_slot < 0 ? opt->d_grad : nullptr;
+		float *ext_gscale = own_gscale ? nullptr : opt->d_gscale;
+		const size_t real_mv = pv->z.mv_bytes;
+
+		adopt(opt, z, pl);
+		pv->z.mv_bytes = real_mv;
+		pv->resident_bytes += 2 * real_mv;
+		opt->d_m = m2;
+		opt->d_v = v2;
+		pv->mv_apart = 1;
+		if (bound_slot >= 0)
+			opt->d_grad = pv->grad_slots + (size_t)bound_slot * pv->grad_slot_bytes;
+		else
+			opt->d_grad = ext_grad;
+		if (ext_gscale)
+			opt->d_gscale = ext_gscale;
+	}
+	(void)hip_ok(hipFree(old_a), "arena hipFree");
+	if (old_b)
+		(void)hip_ok(hipFree(old_b), "arena hipFree");
+	return 0;
+}
+
+extern "C" int anni_adam_set_offload(anni_adam *opt, int on)
+{
+	anni_adam_priv *pv;
+
+	if (!opt || !opt->priv || !device_ready())
+		return -1;
+	pv = opt->priv;
+	if (!on) {
+		pv->offload = 0;
+		return pv->mv_apart ? mv_bring(opt) : 0;
+	}
+	try {
+		if (!pv->h_m && !hip_ok(hipHostMalloc(&pv->h_m, pv->z.mv_bytes, hipHostMallocDefault),
+		    "offload hipHostMalloc")) {
+			(void)hipGetLastError();
+			pv->h_m = nullptr;
+			return -1;
+		}
+		if (!pv->h_v && !hip_ok(hipHostMalloc(&pv->h_v, pv->z.mv_bytes, hipHostMallocDefault),
+		    "offload hipHostMalloc")) {
+			(void)hipGetLastError();
+			pv->h_v = nullptr;
+			return -1;
+		}
+		if (!pv->mv_apart && rehouse_without_mv(opt) != 0)
+			return -1;
+	} catch (...) {
+		return -1;
+	}
+	pv->offload = 1;
+	return mv_send(opt);
+}
+
+extern "C" int anni_adam_mv_on_device(const anni_adam *opt)
+{
+	return opt && opt->d_m && opt->d_v ? 1 : 0;
+}
+
+/* ANN_GNORM_EVERY=N (lm_adam.c:438-450): the gradient norm is computed, and printed every N steps, also when nothing clips. */
+static int gnorm_every(void)
+{
+	static int every = -1;
+
+	if (every < 0) {
+		const char *e = getenv("ANN_GNORM_EVERY");
+
+		every = e ? atoi(e) : 0;
+		if (every < 0)
+			every = 0;
+	}
+	return every;
+}
+
+static int mv_bring(anni_adam *opt);
+static int mv_send(anni_adam *opt);
+
 static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *ev)
 {
 	anni_adam_priv *pv;
@@ -812,6 +1025,7 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 	Flat f;
 	int np = 0;
 	int t;
+	int slot;
 
 	if (!opt || !opt->priv)
 		return -1;
@@ -820,6 +1034,8 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 	if (!opt->d_grad || !device_ready())
 		return -1;
 	pv = opt->priv;
+	if (mv_bring(opt) != 0)			/* offloaded moments come back first (lm_adam.c:295-307) */
+		return -1;
 	st = compute_stream();
 	t = opt->t + 1;				/* lm_adam.c:533; kept only when the step was launched */
 	c.bc1 = 1.0 - pow(opt->beta1, (double)t);	/* lm_adam.c:571-572 */
@@ -838,18 +1054,23 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 	c.lr_wd = c.decay_on ? lr * opt->weight_decay : 0.0;
 	describe(opt, &f);
 	memset(&norm, 0, sizeof(norm));
-	norm.use_norm = (opt->grad_clip > 0.0 || opt->cfg.skip_nonfinite) ? 1 : 0;
+	/* lm_adam.c:466: the norm is wanted for the clip, for the skip, or just to be printed */
+	norm.use_norm = (opt->grad_clip > 0.0 || opt->cfg.skip_nonfinite || gnorm_every() > 0) ? 1 : 0;
 	norm.state = pv->d_state;
 	if (ev && ev[0])
 		(void)hipEventRecord(ev[0], st);
 	if (norm.use_norm) {
 		SumsqFinish fin;
+		int rc;
 
 		fin.ticket = ticket_word(pv);
 		fin.clip = opt->grad_clip > 0.0 ? opt->grad_clip : 0.0;
 		fin.skip_nonfinite = opt->cfg.skip_nonfinite;
 		fin.state = pv->d_state;
-		if (launch_sumsq(st, f, grad_scale, pv->d_partials, &np, &fin) != 0)
+		slot = prof_begin(kProfSumsq, st);
+		rc = launch_sumsq(st, f, grad_scale, pv->d_partials, &np, &fin);
+		prof_end(slot, st);
+		if (rc != 0)
 			return -1;
 	}
 	if (ev && ev[1])
@@ -862,17 +1083,21 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 	if (pv->fp8_twins && launch_fill_bytes(st, pv->d_wamax, 0,
 	    (size_t)opt->n_tensors * sizeof(uint32_t)) != 0)
 		return -1;
+	slot = prof_begin(kProfUpdate, st);
 	if (launch_update(st, f, c, grad_scale, norm) != 0)
 		return -1;
+	prof_end(slot, st);
 	opt->t = t;
 	if (ev && ev[2])
 		(void)hipEventRecord(ev[2], st);
 	if (pv->fp8_twins) {
+		slot = prof_begin(kProfDerived, st);
 		if (launch_amax_fold(st, f, norm.use_norm ? pv->d_state : nullptr) != 0)
 			return -1;
 		if (launch_fp8_twins(st, f, (uint8_t *)opt->d_param_fp8, opt->d_wscale, pv->d_wamax,
 		    opt->n_tensors, norm.use_norm ? pv->d_state : nullptr) != 0)
 			return -1;
+		prof_end(slot, st);
 	}
 	if (ev && ev[3])
 		(void)hipEventRecord(ev[3], st);
@@ -881,6 +1106,10 @@ static int step_impl(anni_adam *opt, double lr, double grad_scale, hipEvent_t *e
 	** them (lm_adam.c:541-547 does this after every device step, a skipped one included).
 	*/
 	gpu_half_wt_invalidate(nullptr);
+	if (pv->offload && mv_send(opt) != 0)	/* lm_adam.c:508-510 */
+		return -1;
+	if (prof_on())
+		gpu_op_prof_dump();		/* lm_adam.c:541 */
 	return 0;
 }
 
@@ -919,16 +1148,10 @@ int anni_adam_sync_stats(anni_adam *opt)
 	** a skipped step always, the norm every ANN_GNORM_EVERY steps.  The step itself never waits
 	** for the host, so they appear when the caller asks for the numbers.
 	*/
-	if (pv->logged_t != opt->t && (opt->grad_clip > 0.0 || opt->cfg.skip_nonfinite)) {
-		static int every = -1;
+	if (pv->logged_t != opt->t
+	    && (opt->grad_clip > 0.0 || opt->cfg.skip_nonfinite || gnorm_every() > 0)) {
+		const int every = gnorm_every();
 
-		if (every < 0) {
-			const char *e = getenv("ANN_GNORM_EVERY");
-
-			every = e ? atoi(e) : 0;
-			if (every < 0)
-				every = 0;
-		}
 		pv->logged_t = opt->t;
 		if (opt->last_skipped)
 			fprintf(stderr, "[adam] step %d skipped: grad norm %g\n", opt->t, opt->last_grad_norm);
@@ -937,105 +1160,6 @@ int anni_adam_sync_stats(anni_adam *opt)
 			    opt->last_clipped ? " (clipped)" : "");
 	}
 	return 0;
-}
-
-static int time_steps_body(anni_adam *opt, int count, void *const *grads, int n_grads,
-	const double *lr, const double *grad_scale, float *ms_total, float *ms_sumsq,
-	float *ms_update)
-{
-	std::vector<hipEvent_t> ev;
-	hipStream_t st;
-	int rc = 0;
-	bool per_kernel = ms_sumsq || ms_update;
-
-	if (!opt || count <= 0 || !lr || !grad_scale || !ms_total || !device_ready())
-		return -1;
-	if (grads && n_grads <= 0)
-		return -1;
-	st = compute_stream();
-	/*
-	** Per kernel: ev[0] before the first step, then per step the events after the sum of squares,
-	** after the update and (only with derived outputs) after those; a step begins where the one
-	** before ended.  Every record costs the stream a few microseconds between two kernels, so
-	** there is none that is not read.
-	*/
-	const bool derived = opt->priv && opt->priv->fp8_twins;
-	const size_t per_step = derived ? 3 : 2;
-
-	ev.resize(per_kernel ? (size_t)count * per_step + 1 : 2);
-	for (size_t i = 0; i < ev.size(); i++)
-		if (hipEventCreate(&ev[i]) != hipSuccess) {
-			for (size_t k = 0; k < i; k++)
-				(void)hipEventDestroy(ev[k]);
-			return -1;
-		}
-	if (!per_kernel)
-		(void)hipEventRecord(ev[0], st);
-	for (int i = 0; i < count && rc == 0; i++) {
-		hipEvent_t four[4] = { nullptr, nullptr, nullptr, nullptr };
-
-		if (per_kernel) {
-			const size_t at = 1 + (size_t)i * per_step;
-
-			four[0] = i == 0 ? ev[0] : nullptr;
-			four[1] = ev[at];
-			four[2] = ev[at + 1];
-			four[3] = derived ? ev[at + 2] : nullptr;
-		}
-		if (grads)
-			(void)anni_adam_bind_grad(opt, grads[i % n_grads]);
-		rc = step_impl(opt, lr[i], grad_scale[i], per_kernel ? four : nullptr);
-		if (rc == 1)
-			rc = -1;		/* a timed run must not contain no-op steps */
-	}
-	if (!per_kernel)
-		(void)hipEventRecord(ev[1], st);
-	if (!hip_ok(sync_stream_and_deliver(), "time_steps sync"))
-		rc = -1;
-	if (rc == 0) {
-		float ms = 0.0f;
-
-		if (per_kernel) {
-			float a = 0.0f, b = 0.0f, d = 0.0f;
-
-			for (int i = 0; i < count; i++) {
-				const size_t at = 1 + (size_t)i * per_step;
-				float x = 0.0f, y = 0.0f, w = 0.0f;
-
-				(void)hipEventElapsedTime(&x, ev[at - 1], ev[at]);
-				(void)hipEventElapsedTime(&y, ev[at], ev[at + 1]);
-				if (derived)
-					(void)hipEventElapsedTime(&w, ev[at + 1], ev[at + 2]);
-				a += x;
-				b += y;
-				d += w;
-			}
-			opt->priv->der_ms = d;
-			(void)hipEventElapsedTime(&ms, ev[0], ev[ev.size() - 1]);
-			if (ms_sumsq)
-				*ms_sumsq = a;
-			if (ms_update)
-				*ms_update = b;
-		} else {
-			(void)hipEventElapsedTime(&ms, ev[0], ev[1]);
-		}
-		*ms_total = ms;
-	}
-	for (size_t i = 0; i < ev.size(); i++)
-		(void)hipEventDestroy(ev[i]);
-	return rc;
-}
-
-int anni_adam_time_steps(anni_adam *opt, int count, void *const *grads, int n_grads,
-	const double *lr, const double *grad_scale, float *ms_total, float *ms_sumsq,
-	float *ms_update)
-{
-	try {
-		return time_steps_body(opt, count, grads, n_grads, lr, grad_scale, ms_total, ms_sumsq,
-		    ms_update);
-	} catch (...) {
-		return -1;
-	}
 }
 
 /* ---- optimizer block of a checkpoint (lang/lm_serialize.c:263-331,526-587) ----------- */
@@ -1190,7 +1314,7 @@ int anni_adam_export_mv(anni_adam *opt, int64_t first, int64_t count, float *pai
 		return -1;
 	io.mem = pairs;
 	io.fd = -1;
-	return export_pairs(opt, first, count, io);
+	return with_moments(opt, [&] { return export_pairs(opt, first, count, io); });
 }
 
 int anni_adam_import_mv(anni_adam *opt, int64_t first, int64_t count, const float *pairs)
@@ -1202,7 +1326,7 @@ int anni_adam_import_mv(anni_adam *opt, int64_t first, int64_t count, const floa
 		return -1;
 	io.mem = const_cast<float *>(pairs);
 	io.fd = -1;
-	return import_pairs(opt, first, count, io);
+	return with_moments(opt, [&] { return import_pairs(opt, first, count, io); });
 }
 
 static int write_all(int fd, const void *buf, size_t n)
@@ -1251,7 +1375,7 @@ int anni_adam_write_state(anni_adam *opt, int fd, int epoch, int step)
 		return -1;
 	io.mem = nullptr;
 	io.fd = fd;
-	return export_pairs(opt, 0, opt->n, io);	/* write(2) straight from the page-locked buffers */
+	return with_moments(opt, [&] { return export_pairs(opt, 0, opt->n, io); });	/* write(2) straight from the page-locked buffers */
 }
 
 int anni_adam_read_state(anni_adam *opt, int fd, int *epoch, int *step)
@@ -1265,7 +1389,7 @@ int anni_adam_read_state(anni_adam *opt, int fd, int *epoch, int *step)
 		return -1;		/* lm_serialize.c:546-562: has_adam == 1 and the same slot count */
 	io.mem = nullptr;
 	io.fd = fd;
-	if (import_pairs(opt, 0, opt->n, io) != 0)
+	if (with_moments(opt, [&] { return import_pairs(opt, 0, opt->n, io); }) != 0)
 		return -1;		/* a short file: the moments read so far are in place, t is not */
 	opt->t = head[3];		/* so the learning-rate schedule continues (lm_serialize.c:564) */
 	if (epoch)
@@ -1347,9 +1471,21 @@ void anni_gpu_flush(void)
 		(void)compute_stream();		/* launches the pending batch of small copies, if any */
 }
 
-void anni_gpu_reload_switches(void)
+/* ---- what libanni_bench.so needs from inside this library (anni_hooks.h) ------------------ */
+
+int anni_hook_step_events(anni_adam *opt, double lr, double grad_scale, void *const events[4])
+{
+	return step_impl(opt, lr, grad_scale, (hipEvent_t *)events);
+}
+
+void anni_hook_reload_switches(void)
 {
 	reload_switches();
+}
+
+void anni_hook_fold_guard_stats(int *runs, int *mismatches)
+{
+	fold_guard_stats(runs, mismatches);
 }
 
 int anni_gpu_device_info(char *name, size_t cap, int *driver_version)

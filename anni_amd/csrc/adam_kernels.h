@@ -122,13 +122,18 @@ struct SumsqFinish {
 /* Reads the ANNI_* tuning switches from the environment again (they are read once, on first use). */
 void	reload_switches(void);
 
+/* How often the self-check of launch_sumsq's second stage has run in this process, and how often its two forms disagreed. */
+void	fold_guard_stats(int *runs, int *mismatches);
+
 /* Workgroups of a resident grid for a flat of n elements on the current device. */
 int	grid_for(int64_t n);
 
 /*
 ** partials[0..*n_partials) = per-workgroup sums of (g * grad_scale)^2, fixed order.  With `fin`
 ** the last workgroup to finish also folds them in index order into fin->state = {sum, sqrt,
-** clip-adjusted scale, flags}.
+** clip-adjusted scale, flags}.  The first such call on a device (and the first after
+** reload_switches) launches the sum twice more and waits for the stream once: the self-check of
+** the second stage (adam_kernels.hip, fold_guard); every other call is asynchronous.
 */
 int	launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *partials,
 		int *n_partials, const SumsqFinish *fin);

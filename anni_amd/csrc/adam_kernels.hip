@@ -11,8 +11,11 @@
 */
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <atomic>
+#include <mutex>
 #include "adam_kernels.h"
 
 namespace anni {
@@ -1221,6 +1224,7 @@ struct Switches {
 	int	fold_fence;	/* ANNI_FOLD=fence: the norm's second stage takes the partials over with fences (see sumsq_finish) */
 };
 static Switches g_sw;
+static void fold_guard_reset(void);
 
 void reload_switches(void)
 {
@@ -1237,6 +1241,7 @@ void reload_switches(void)
 		g_sw.fold_fence = (e && strcmp(e, "fence") == 0) ? 1 : 0;
 	}
 	g_sw.loaded = 1;
+	fold_guard_reset();
 }
 
 static const Switches &sw(void)
@@ -1323,8 +1328,9 @@ static int check_flat(const Flat &f, bool need_state)
 	return 0;
 }
 
-int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *partials,
-	int *n_partials, const SumsqFinish *fin)
+/* fence: 1 = the second stage takes the partials over with fences, 0 = with atomic accesses. */
+static int sumsq_launch(hipStream_t st, const Flat &f, double grad_scale, double *partials,
+	int *n_partials, const SumsqFinish *fin, int fence)
 {
 	SumsqArgs a;
 	int grid;
@@ -1363,7 +1369,7 @@ int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *parti
 	a.clip = 0.0;
 	a.skip_nonfinite = 0;
 	a.state = nullptr;
-	a.fence = sw().fold_fence;
+	a.fence = fence;
 	if (fin) {
 		if (!fin->ticket || !fin->state || !aligned(fin->ticket, 128))
 			return -1;
@@ -1399,6 +1405,99 @@ int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *parti
 #undef SUMSQ_LAUNCH
 	*n_partials = grid;
 	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+/*
+** Self-check of the second stage.  The default hand-over of the partials (atomic accesses, see
+** sumsq_finish) leans on how gfx950 performs device-scope atomics, which the HIP memory model
+** does not promise; the fenced form leans on nothing.  So the first sum of squares with a second
+** stage on each device -- and the first after the switches were read again -- runs both forms on
+** the caller's own gradient flat and grid before anything consumes a result, waits, and compares
+** the two step states bit for bit.  If they differ the process goes over to the fenced form for
+** good and says so once on stderr.  Cost: two extra launches and one stream synchronisation per
+** process and device.  A stream under capture cannot be waited for: there the check is put off
+** until the first launch outside a capture.
+*/
+static const int kGuardDevices = 64;
+static std::atomic<int> g_fold_checked[kGuardDevices];
+static std::mutex g_fold_mu;
+static StepState *g_fold_host;		/* page-locked, two states */
+static int g_fold_runs;
+static int g_fold_mismatches;
+
+static void fold_guard_reset(void)
+{
+	for (int i = 0; i < kGuardDevices; i++)
+		g_fold_checked[i].store(0, std::memory_order_relaxed);
+}
+
+void fold_guard_stats(int *runs, int *mismatches)
+{
+	std::lock_guard<std::mutex> lk(g_fold_mu);
+
+	if (runs)
+		*runs = g_fold_runs;
+	if (mismatches)
+		*mismatches = g_fold_mismatches;
+}
+
+static void fold_guard(hipStream_t st, const Flat &f, double grad_scale, double *partials,
+	const SumsqFinish *fin)
+{
+	hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+	SumsqFinish mine;
+	int dev = -1;
+	int np = 0;
+
+	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kGuardDevices) {
+		(void)hipGetLastError();
+		return;
+	}
+	if (g_fold_checked[dev].load(std::memory_order_acquire))
+		return;
+	if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
+		(void)hipGetLastError();
+		return;
+	}
+	std::lock_guard<std::mutex> lk(g_fold_mu);
+
+	if (g_fold_checked[dev].load(std::memory_order_relaxed))
+		return;
+	if (!g_fold_host && hipHostMalloc((void **)&g_fold_host, 2 * sizeof(StepState),
+	    hipHostMallocPortable) != hipSuccess) {
+		(void)hipGetLastError();
+		g_fold_host = nullptr;
+		return;
+	}
+	memset(g_fold_host, 0xff, 2 * sizeof(StepState));
+	mine = *fin;
+	for (int fence = 0; fence < 2; fence++) {
+		mine.state = g_fold_host + fence;
+		if (sumsq_launch(st, f, grad_scale, partials, &np, &mine, fence) != 0)
+			return;
+	}
+	if (hipStreamSynchronize(st) != hipSuccess) {
+		(void)hipGetLastError();
+		return;
+	}
+	g_fold_runs++;
+	if (memcmp(&g_fold_host[0], &g_fold_host[1], sizeof(StepState)) != 0) {
+		g_fold_mismatches++;
+		g_sw.fold_fence = 1;
+		fprintf(stderr, "[anni] sum of squares: the atomic and the fenced hand-over of the partials "
+		    "disagree on this device (sum %.17g against %.17g over %d workgroups); "
+		    "using the fenced one from now on\n", g_fold_host[0].sumsq, g_fold_host[1].sumsq, np);
+	}
+	g_fold_checked[dev].store(1, std::memory_order_release);
+}
+
+int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *partials,
+	int *n_partials, const SumsqFinish *fin)
+{
+	if (fin && fin->ticket && fin->state && !sw().fold_fence && check_flat(f, false) == 0
+	    && partials)
+		fold_guard(st, f, grad_scale, partials, fin);
+	return sumsq_launch(st, f, grad_scale, partials, n_partials, fin, sw().fold_fence);
 }
 
 #ifndef ANNI_UPDATE_UNROLL

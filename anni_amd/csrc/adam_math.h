@@ -40,18 +40,21 @@ struct Elem {
 };
 
 /*
-** a / b for a step constant b whose correctly rounded reciprocal rb the host supplies:
-** q = a*rb, then one exact residual a - b*q folded back.  The result is a/b rounded to
-** nearest unless a/b lies within ~2^-52 ulp of a rounding boundary (then it may be the
-** other neighbour): about one quotient in 2^52.  Not for an infinite a: the residual would be
-** inf - inf (adam_elem sends those to the IEEE division).  Used only where the update is bound
-** by arithmetic (narrow storage types); the all-f32 mode keeps the IEEE division.
+** a / b for a step constant b > 0 whose correctly rounded reciprocal rb the host supplies:
+** q = a*rb, then one exact residual a - b*q folded back.  The result is a/b rounded to nearest
+** unless a/b lies within ~2^-52 ulp of a rounding boundary (then it may be the other neighbour).
+** Compared on the host with the IEEE quotient for b = 1 - beta^t, beta in {0.9, 0.95, 0.999},
+** t = 1..10000, over 10^8 float-valued numerators from every binary exponent: no difference
+** (tests/c/div_by_const_test.c).  The residual of a zero is +0 whatever the zero's sign, so the
+** sign is put back: -0 / b is -0.  Not for an infinite a: the residual would be inf - inf
+** (adam_elem sends those to the IEEE division).  Used only where the update is bound by
+** arithmetic (narrow storage types); the all-f32 mode keeps the IEEE division.
 */
 __device__ __forceinline__ double div_by_const(double a, double b, double rb)
 {
 	const double q = a * rb;
 
-	return __builtin_fma(__builtin_fma(-b, q, a), rb, q);
+	return __builtin_copysign(__builtin_fma(__builtin_fma(-b, q, a), rb, q), a);
 }
 
 /*

@@ -30,5 +30,15 @@ bool		hip_ok(hipError_t err, const char *what);
 */
 bool		release_idle_pools(void);
 
+/*
+** ANN_OP_PROF=1 (num/gpu_cuda.cu:3205-3409): an event pair around an operation of the optimizer
+** step, summed per kind and printed by gpu_op_prof_dump.  prof_begin records the first event on
+** `st` and returns the pair's slot (-1: profiling is off), prof_end records the second.
+*/
+enum { kProfSumsq = 0, kProfUpdate = 1, kProfDerived = 2, kProfKinds = 3 };
+bool		prof_on(void);
+int		prof_begin(int kind, hipStream_t st);
+void		prof_end(int slot, hipStream_t st);
+
 } /* namespace anni */
 #endif

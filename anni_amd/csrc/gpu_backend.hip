@@ -15,6 +15,7 @@
 #include "adam_kernels.h"
 #include "anni_gpu.h"
 #include "backend_state.h"
+#include "busy_flag.h"
 #include "placement.h"
 #include "pool_chunks.h"
 
@@ -92,14 +93,17 @@ bool hip_ok(hipError_t err, const char *what)
 /*
 ** lang/lm_adam.c moves every bias / LayerNorm vector with its own gpu_memcpy_h2d before the
 ** step and its own gpu_memcpy_d2h_async after it (lm_adam.c:372-377,407-413): 146 + 73 copies
-** of a few KiB per step at the reference's 185M size, more time than the two kernels.  Copies
-** of kSmallCopy bytes or less are therefore batched: an H2D is copied into a page-locked
-** staging ring at once (the caller may reuse its buffer on return, as with a pageable
-** cudaMemcpyAsync) and described in a table; the next operation on the stream first launches
-** ONE kernel that moves the whole batch.  A small async D2H is gathered the same way into the
-** ring and handed to its host destination at the next synchronisation, which is when the
-** contract makes it visible (num/gpu.h:44-47).  Order on the stream is kept because every
-** entry point flushes the pending batch before it enqueues anything.
+** of a few KiB per step at the reference's 185M size (170 + 85 at 555M, the head bias of 400 KB
+** among them), more time than the two kernels when each is a copy of its own.  Copies of
+** kSmallCopy bytes or less are therefore batched: an H2D is copied into a page-locked staging
+** ring at once (the caller may reuse its buffer on return, as with a pageable cudaMemcpyAsync)
+** and described in a table, one entry per piece of kPieceBytes; a kernel with one workgroup per
+** piece moves the batch.  That kernel is launched as soon as kFlushBytes are waiting -- it pulls
+** them over the host link while the caller is still staging the next vectors -- and at the
+** latest by the next operation on the stream.  A small async D2H is gathered the same way into
+** the ring and handed to its host destination at the next synchronisation, which is when the
+** contract makes it visible (num/gpu.h:44-47).  Order on the stream is kept because every entry
+** point puts the pending batch on the stream before it enqueues anything.
 ** ANNI_SMALL_COPY_BATCH=0 switches the batching off.
 */
 struct CopyDesc {
@@ -108,7 +112,9 @@ struct CopyDesc {
 	unsigned long long	nbytes;
 };
 
-static const size_t kSmallCopy = (size_t)64 << 10;
+static const size_t kSmallCopy = (size_t)1 << 20;
+static const size_t kPieceBytes = (size_t)16 << 10;	/* a multiple of 16: every piece keeps the copy's alignment */
+static const size_t kFlushBytes = (size_t)256 << 10;
 static const size_t kStageBytes = (size_t)16 << 20;
 static const int kDescSlots = 8192;
 static char *g_stage;			/* page-locked, device-visible */
@@ -116,6 +122,7 @@ static CopyDesc *g_desc;		/* page-locked, device-visible */
 static size_t g_stage_used;		/* bump pointers; reset after every full synchronisation */
 static int g_desc_used;
 static int g_batch_first;		/* descriptors [g_batch_first, g_desc_used) are not launched yet */
+static size_t g_batch_bytes;		/* what they move */
 /* g_batch_dir (declared above): 0 none, 1 host-to-device, 2 device-to-host */
 struct Delivery {
 	void	*host;
@@ -126,11 +133,12 @@ static Delivery g_deliver[kDescSlots];	/* gathered D2H data waiting for a synchr
 static int g_deliver_n;
 
 /*
-** One workgroup per copy.  The staging side of every copy is placed at the same offset from
+** One workgroup per piece.  The staging side of every copy is placed at the same offset from
 ** a 16-byte boundary as its device side (batch_add_locked), so after at most 15 leading bytes
-** both run in 16-byte steps: a bias / LayerNorm vector of a few KiB is one load and one store
-** per lane, all in flight together.  (Byte by byte the same batch spent 0.3 ms of a 1.6 ms
-** step waiting on the host link, one round trip after the other.)
+** both run in 16-byte steps, four of them in flight per lane: a bias / LayerNorm vector of a few
+** KiB is one round, a long vector is spread over many workgroups.  (Byte by byte the same batch
+** spent 0.3 ms of a 1.6 ms step waiting on the host link, one round trip after the other; one
+** workgroup per 400 KB vector pulled it at a third of the link's rate.)
 */
 __global__ __launch_bounds__(256) void small_copy_kernel(const CopyDesc *desc, char *stage,
 	int to_device)
@@ -144,11 +152,27 @@ __global__ __launch_bounds__(256) void small_copy_kernel(const CopyDesc *desc, c
 	const size_t head = lead < d.nbytes ? lead : d.nbytes;
 	const size_t body = (d.nbytes - head) / 16;
 	const size_t tail = head + body * 16;
+	const uint4 *s16 = (const uint4 *)(src + head);
+	uint4 *d16 = (uint4 *)(dst + head);
 
+	static_assert(kPieceBytes == 4 * 256 * 16, "a piece is four 16-byte accesses per lane");
 	if (threadIdx.x < head)
 		dst[threadIdx.x] = src[threadIdx.x];
-	for (size_t i = threadIdx.x; i < body; i += 256)
-		((uint4 *)(dst + head))[i] = ((const uint4 *)(src + head))[i];
+	if (body >= 1024) {
+		uint4 w[4];
+
+#pragma unroll
+		for (int u = 0; u < 4; u++)
+			w[u] = s16[threadIdx.x + u * 256];
+#pragma unroll
+		for (int u = 0; u < 4; u++)
+			d16[threadIdx.x + u * 256] = w[u];
+		for (size_t i = 1024 + threadIdx.x; i < body; i += 256)
+			d16[i] = s16[i];
+	} else {
+		for (size_t i = threadIdx.x; i < body; i += 256)
+			d16[i] = s16[i];
+	}
 	if (tail + threadIdx.x < d.nbytes)
 		dst[tail + threadIdx.x] = src[tail + threadIdx.x];
 }
@@ -189,6 +213,7 @@ static void batch_flush_locked(void)
 		(void)hip_ok_locked(hipGetLastError(), "small copy batch");
 	}
 	g_batch_first = g_desc_used;
+	g_batch_bytes = 0;
 	g_batch_dir = 0;
 }
 
@@ -201,6 +226,7 @@ static void batch_deliver_locked(void)
 	g_stage_used = 0;
 	g_desc_used = 0;
 	g_batch_first = 0;
+	g_batch_bytes = 0;
 }
 
 /* Queues one small copy; false = does not qualify (the caller copies the ordinary way).  g_mu held. */
@@ -208,12 +234,14 @@ static bool batch_add_locked(int dir, void *dev, void *host, size_t nbytes)
 {
 	const size_t skew = (uintptr_t)dev & 15;	/* staging keeps the device side's alignment */
 	const size_t need = (skew + nbytes + 255) / 256 * 256;
+	const int pieces = (int)((nbytes + kPieceBytes - 1) / kPieceBytes);
+	size_t at;
 
 	if (nbytes > kSmallCopy || !batch_on())
 		return false;
 	if (g_batch_dir != 0 && g_batch_dir != dir)
 		batch_flush_locked();
-	if (g_stage_used + need > kStageBytes || g_desc_used == kDescSlots
+	if (g_stage_used + need > kStageBytes || g_desc_used + pieces > kDescSlots
 	    || g_deliver_n == kDescSlots) {
 		/* rings full: drain everything, then start over */
 		batch_flush_locked();
@@ -221,20 +249,27 @@ static bool batch_add_locked(int dir, void *dev, void *host, size_t nbytes)
 			return false;
 		batch_deliver_locked();
 	}
-	g_desc[g_desc_used].dev = dev;
-	g_desc[g_desc_used].stage_off = g_stage_used + skew;
-	g_desc[g_desc_used].nbytes = nbytes;
+	at = g_stage_used + skew;
+	for (size_t done = 0; done < nbytes; done += kPieceBytes) {
+		g_desc[g_desc_used].dev = (char *)dev + done;
+		g_desc[g_desc_used].stage_off = at + done;
+		g_desc[g_desc_used].nbytes = nbytes - done < kPieceBytes ? nbytes - done : kPieceBytes;
+		g_desc_used++;
+	}
 	if (dir == 1) {
-		memcpy(g_stage + g_stage_used + skew, host, nbytes);
+		memcpy(g_stage + at, host, nbytes);
 	} else {
 		g_deliver[g_deliver_n].host = host;
-		g_deliver[g_deliver_n].stage_off = g_stage_used + skew;
+		g_deliver[g_deliver_n].stage_off = at;
 		g_deliver[g_deliver_n].nbytes = nbytes;
 		g_deliver_n++;
 	}
-	g_desc_used++;
 	g_stage_used += need;
+	g_batch_bytes += nbytes;
 	g_batch_dir = dir;
+	/* enough for a launch of its own: the device pulls it while the caller stages the next vectors */
+	if (dir == 1 && g_batch_bytes >= kFlushBytes)
+		batch_flush_locked();
 	return true;
 }
 
@@ -311,18 +346,27 @@ static bool scratch_ready(void)
 
 /* ---- ANN_OP_PROF=1: event pairs around the step's launches ---------------- */
 
+/*
+** The reference times every backend operation with an event pair and prints the table from
+** gpu_op_prof_dump, which lm_adam_step_scaled calls after each device step
+** (num/gpu_cuda.cu:3205-3409, lang/lm_adam.c:541).  Here the operations are the optimizer's:
+** the sum of squares, the update, and the passes that keep derived weight copies current.
+** Pairs are resolved at gpu_device_sync and at the dump.  The table and its slots are guarded
+** by g_mu; the events themselves are recorded on the compute stream outside it.
+*/
 struct ProfSlot {
 	hipEvent_t	a;
 	hipEvent_t	b;
-	int		kind;	/* 0 sumsq, 1 update */
+	int		kind;
 };
-#define PROF_SLOTS 64
+#define PROF_SLOTS 256
 static ProfSlot g_prof[PROF_SLOTS];
 static int g_prof_n;
-static double g_prof_ms[2];
-static int g_prof_calls[2];
+static int g_prof_round;		/* counts resolutions: a slot number is only good within its round */
+static double g_prof_ms[kProfKinds];
+static int g_prof_calls[kProfKinds];
 
-static bool prof_on(void)
+bool prof_on(void)
 {
 	static int on = -1;
 
@@ -334,49 +378,74 @@ static bool prof_on(void)
 	return on == 1;
 }
 
-static void prof_resolve(void)
+/* g_mu held.  Waits for the recorded pairs (the stream has to reach them) and adds them to the table. */
+static void prof_resolve_locked(void)
 {
 	for (int i = 0; i < g_prof_n; i++) {
 		float ms = 0.0f;
 
-		if (hipEventSynchronize(g_prof[i].b) == hipSuccess
+		if (g_prof[i].b && hipEventSynchronize(g_prof[i].b) == hipSuccess
 		    && hipEventElapsedTime(&ms, g_prof[i].a, g_prof[i].b) == hipSuccess) {
 			g_prof_ms[g_prof[i].kind] += ms;
 			g_prof_calls[g_prof[i].kind]++;
 		}
 		(void)hipEventDestroy(g_prof[i].a);
-		(void)hipEventDestroy(g_prof[i].b);
+		if (g_prof[i].b)
+			(void)hipEventDestroy(g_prof[i].b);
 	}
+	(void)hipGetLastError();
 	g_prof_n = 0;
+	g_prof_round = (g_prof_round + 1) & 0xffff;
 }
 
-struct ProfScope {
-	int	slot;
+/* The first event of a pair, recorded on `st`; the pair's slot, or -1 (profiling off, no slot). */
+int prof_begin(int kind, hipStream_t st)
+{
+	hipEvent_t a = nullptr;
+	int slot;
 
-	explicit ProfScope(int kind) : slot(-1)
+	if (!prof_on() || kind < 0 || kind >= kProfKinds)
+		return -1;
+	if (hipEventCreate(&a) != hipSuccess) {
+		(void)hipGetLastError();
+		return -1;
+	}
 	{
-		if (!prof_on())
-			return;
+		std::lock_guard<std::mutex> lk(g_mu);
+
 		if (g_prof_n == PROF_SLOTS)
-			prof_resolve();
-		ProfSlot &s = g_prof[g_prof_n];
-
-		if (hipEventCreate(&s.a) != hipSuccess)
-			return;
-		if (hipEventCreate(&s.b) != hipSuccess) {
-			(void)hipEventDestroy(s.a);
-			return;
-		}
-		s.kind = kind;
-		(void)hipEventRecord(s.a, g_stream);
+			prof_resolve_locked();
 		slot = g_prof_n++;
+		g_prof[slot].a = a;
+		g_prof[slot].b = nullptr;
+		g_prof[slot].kind = kind;
+		slot += g_prof_round * PROF_SLOTS;
 	}
-	~ProfScope()
-	{
-		if (slot >= 0)
-			(void)hipEventRecord(g_prof[slot].b, g_stream);
+	(void)hipEventRecord(a, st);
+	return slot;
+}
+
+/* The second event of the pair `slot` (a result of prof_begin that the table has not resolved since). */
+void prof_end(int slot, hipStream_t st)
+{
+	hipEvent_t b = nullptr;
+
+	if (slot < 0)
+		return;
+	if (hipEventCreate(&b) != hipSuccess) {
+		(void)hipGetLastError();
+		return;
 	}
-};
+	(void)hipEventRecord(b, st);
+	std::lock_guard<std::mutex> lk(g_mu);
+
+	/* a table that was resolved in between has dropped the pair: nothing to complete */
+	if (slot / PROF_SLOTS == g_prof_round && slot % PROF_SLOTS < g_prof_n
+	    && !g_prof[slot % PROF_SLOTS].b)
+		g_prof[slot % PROF_SLOTS].b = b;
+	else
+		(void)hipEventDestroy(b);
+}
 
 } /* namespace anni */
 
@@ -433,7 +502,7 @@ void gpu_device_sync(void)
 		(void)hip_ok(err, "hipDeviceSynchronize");
 	} else if (prof_on()) {
 		std::lock_guard<std::mutex> lk(g_mu);
-		prof_resolve();
+		prof_resolve_locked();
 	}
 }
 
@@ -467,13 +536,13 @@ const char *gpu_debug_last_error(void)
 
 void gpu_op_prof_dump(void)
 {
-	static const char *name[2] = { "grad_sumsq", "adam_step" };
+	static const char *name[kProfKinds] = { "grad_sumsq", "adam_step", "derived" };
 
 	if (!prof_on() || !device_ready())
 		return;
 	std::lock_guard<std::mutex> lk(g_mu);
-	prof_resolve();
-	for (int k = 0; k < 2; k++) {
+	prof_resolve_locked();
+	for (int k = 0; k < kProfKinds; k++) {
 		if (!g_prof_calls[k])
 			continue;
 		fprintf(stderr, "[op-prof] %-12s %8.3f ms  %d calls\n", name[k], g_prof_ms[k],
@@ -906,6 +975,14 @@ void gpu_adam_set_weight_decay(double wd)
 	g_wd = wd > 0.0 ? wd : 0.0;
 }
 
+/*
+** One result slot, one partials array and one set of ticket words serve every call (as the
+** reference's static accumulator does, num/gpu_cuda.cu:8485-8486): a call that arrives while
+** another is between its launch and its read-back would fold the other's partials or read the
+** other's result, so it is turned away (-1: the caller takes its CPU path) instead.
+*/
+static BusyFlag g_sumsq_busy;
+
 int gpu_grad_sumsq(const ann_real *d_x, int n, double *out)
 {
 	Flat f;
@@ -913,22 +990,28 @@ int gpu_grad_sumsq(const ann_real *d_x, int n, double *out)
 
 	if (!d_x || n <= 0 || !out || !device_ready() || !scratch_ready())
 		return -1;
+	BusyScope only(g_sumsq_busy);
+
+	if (!only.entered)
+		return -1;
 	memset(&f, 0, sizeof(f));
 	f.g = (void *)d_x;
 	f.n = n;
 	f.grad_type = kF32;
 	(void)stream_for_op();
 	{
-		ProfScope prof(0);
-
+		const int slot = prof_begin(kProfSumsq, g_stream);
 		SumsqFinish fin;
+		int rc;
 
 		/* the second stage stores its result straight into page-locked host memory */
 		fin.ticket = (unsigned int *)(g_partials + kMaxPartials);
 		fin.clip = 0.0;
 		fin.skip_nonfinite = 0;
 		fin.state = g_host_state;
-		if (launch_sumsq(g_stream, f, 1.0, g_partials, &np, &fin) != 0)
+		rc = launch_sumsq(g_stream, f, 1.0, g_partials, &np, &fin);
+		prof_end(slot, g_stream);
+		if (rc != 0)
 			return -1;
 	}
 	if (!hip_ok(sync_stream_and_deliver(), "sumsq sync"))
@@ -975,9 +1058,13 @@ int gpu_adam_step_dev_bf16(ann_real *d_param, void *d_param_bf16, ann_real *d_gr
 	f.uniform_flags = (g_wd > 0.0 ? kSegDecay : 0u) | (f.twin ? kSegTwin : 0u);
 	memset(&norm, 0, sizeof(norm));
 	(void)stream_for_op();
-	ProfScope prof(1);
+	{
+		const int slot = prof_begin(kProfUpdate, g_stream);
+		const int rc = launch_update(g_stream, f, c, grad_scale, norm);
 
-	return launch_update(g_stream, f, c, grad_scale, norm);
+		prof_end(slot, g_stream);
+		return rc;
+	}
 }
 
 } /* extern "C" */

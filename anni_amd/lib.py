@@ -1,6 +1,7 @@
-"""ctypes loader of libanni_gpu_hip.so.
+"""ctypes loader of libanni_gpu_hip.so (the product) and libanni_bench.so (the measuring and
+testing utilities of include/anni_bench.h, a library of its own linked against the product).
 
-There is no CPU fallback: if the library has not been built, loading raises
+There is no CPU fallback: if the libraries have not been built, loading raises
 ``LibraryMissing`` and nothing in this package computes anything.
 """
 import ctypes as C
@@ -8,6 +9,7 @@ import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(HERE, "libanni_gpu_hip.so")
+BENCH_SO_PATH = os.path.join(HERE, "libanni_bench.so")
 
 F32, BF16, FP8_E4M3 = 0, 1, 2
 T_DECAY, T_TWIN, T_FP8TWIN = 1, 2, 4
@@ -101,24 +103,20 @@ _PROTOS = {
     "anni_adam_bind_grad": (C.c_int, [C.POINTER(Adam), C.c_void_p]),
     "anni_adam_seed_twins": (C.c_int, [C.POINTER(Adam)]),
     "anni_adam_zero_grad": (C.c_int, [C.POINTER(Adam)]),
+    "anni_adam_set_offload": (C.c_int, [C.POINTER(Adam), C.c_int]),
+    "anni_adam_mv_on_device": (C.c_int, [C.POINTER(Adam)]),
     "anni_adam_quantize_grads": (C.c_int, [C.POINTER(Adam), C.c_void_p]),
     "anni_adam_quantize_grads_static": (C.c_int, [C.POINTER(Adam), C.c_void_p]),
     "anni_adam_step_scaled": (C.c_int, [C.POINTER(Adam), C.c_double, C.c_double]),
     "anni_adam_step": (C.c_int, [C.POINTER(Adam), C.c_double]),
     "anni_adam_sync_stats": (C.c_int, [C.POINTER(Adam)]),
-    "anni_adam_time_steps": (C.c_int, [C.POINTER(Adam), C.c_int, C.POINTER(C.c_void_p),
-                                       C.c_int, C.POINTER(C.c_double),
-                                       C.POINTER(C.c_double), C.POINTER(C.c_float),
-                                       C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "anni_adam_export_mv": (C.c_int, [C.POINTER(Adam), C.c_int64, C.c_int64, C.c_void_p]),
     "anni_adam_import_mv": (C.c_int, [C.POINTER(Adam), C.c_int64, C.c_int64, C.c_void_p]),
     "anni_adam_write_state": (C.c_int, [C.POINTER(Adam), C.c_int, C.c_int, C.c_int]),
     "anni_adam_read_state": (C.c_int, [C.POINTER(Adam), C.c_int, C.POINTER(C.c_int),
                                        C.POINTER(C.c_int)]),
     "anni_adam_enable_derived": (C.c_int, [C.POINTER(Adam), C.POINTER(Pack), C.c_int, C.c_int64]),
-    "anni_adam_timed_derived_ms": (C.c_float, [C.POINTER(Adam)]),
     "anni_gpu_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int)]),
-    "anni_gpu_reload_switches": (None, []),
     "anni_lr_set_schedule": (None, [C.c_int, C.c_int, C.c_char_p]),
     "anni_lr_set_sched_from": (None, [C.c_int]),
     "anni_lr_set_override": (None, [C.c_double]),
@@ -126,16 +124,39 @@ _PROTOS = {
     "anni_gpu_stream": (C.c_void_p, []),
     "anni_gpu_set_stream": (None, [C.c_void_p]),
     "anni_gpu_flush": (None, []),
-    "anni_fill_normal_f32": (C.c_int, [C.c_void_p, C.c_int64, C.c_uint64, C.c_uint64,
-                                       C.c_float, C.c_float]),
-    "anni_copy_bytes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "anni_f32_to_bf16": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64]),
     "anni_fp8_quantize": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]),
     "anni_colsum_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]),
     "anni_colsum_add_batch": (C.c_int, [C.POINTER(Colsum), C.c_int]),
 }
 
+# include/anni_bench.h (libanni_bench.so)
+_BENCH_PROTOS = {
+    "anni_adam_time_steps": (C.c_int, [C.POINTER(Adam), C.c_int, C.POINTER(C.c_void_p),
+                                       C.c_int, C.POINTER(C.c_double),
+                                       C.POINTER(C.c_double), C.POINTER(C.c_float),
+                                       C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+    "anni_adam_timed_derived_ms": (C.c_float, [C.POINTER(Adam)]),
+    "anni_gpu_reload_switches": (None, []),
+    "anni_fill_normal_f32": (C.c_int, [C.c_void_p, C.c_int64, C.c_uint64, C.c_uint64,
+                                       C.c_float, C.c_float]),
+    "anni_copy_bytes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "anni_fold_guard_stats": (C.c_int, [C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+}
+
 _lib = None
+
+
+class _Both:
+    """The product library with the bench library's entry points beside it: one object to call."""
+
+    def __init__(self, product, bench):
+        self._product, self._bench = product, bench
+
+    def __getattr__(self, name):
+        if name in _BENCH_PROTOS:
+            return getattr(self._bench, name)
+        return getattr(self._product, name)
 
 
 def load():
@@ -146,12 +167,16 @@ def load():
             raise LibraryMissing(
                 "%s is missing: build it with `make -C anni_amd/csrc` "
                 "(or __graft_entry__.build()); there is no CPU fallback" % SO_PATH)
-        L = C.CDLL(SO_PATH)
-        for name, (res, args) in _PROTOS.items():
-            fn = getattr(L, name)
-            fn.restype = res
-            fn.argtypes = args
-        _lib = L
+        if not os.path.exists(BENCH_SO_PATH):
+            raise LibraryMissing("%s is missing: build it with `make -C anni_amd/csrc`" % BENCH_SO_PATH)
+        L = C.CDLL(SO_PATH, mode=C.RTLD_GLOBAL)
+        B = C.CDLL(BENCH_SO_PATH)
+        for lib_, protos in ((L, _PROTOS), (B, _BENCH_PROTOS)):
+            for name, (res, args) in protos.items():
+                fn = getattr(lib_, name)
+                fn.restype = res
+                fn.argtypes = args
+        _lib = _Both(L, B)
     return _lib
 
 

@@ -70,7 +70,7 @@ typedef struct anni_adam_config {
 	int	twins;		/* 1: allocate the bf16 twin flat */
 	int	skip_nonfinite;	/* 1: a non-finite gradient norm skips the update (lm_adam.c:474-483) */
 	int	grad_slots;	/* gradient flats the arena allocates (slot 0 starts bound); 0: bind one with anni_adam_bind_grad */
-	int	layout;		/* ANNI_LAYOUT_AUTO / _COMPACT / _SPREAD */
+	int	layout;		/* ANNI_LAYOUT_AUTO / _COMPACT / _SPLIT */
 } anni_adam_config;
 
 /*
@@ -196,12 +196,30 @@ int	anni_adam_quantize_grads(anni_adam *opt, const float *d_src);
 int	anni_adam_quantize_grads_static(anni_adam *opt, const float *d_src);
 /*
 ** lm_adam_step_scaled (lm_adam.c:522-607): lr <= 0 returns 1 without advancing t;
-** otherwise t++, [sum of squares when grad_clip > 0 or skip_nonfinite], update.
-** Asynchronous on the compute stream: nothing is read back.
+** otherwise t++, [sum of squares when grad_clip > 0, skip_nonfinite or ANN_GNORM_EVERY > 0,
+** lm_adam.c:466], update.  Asynchronous on the compute stream: nothing is read back.  Two
+** exceptions: the very first sum of squares on a device waits for the stream once (a self-check
+** of its second stage), and with ANN_OP_PROF=1 every step ends with the reference's
+** gpu_op_prof_dump (lm_adam.c:541), which waits for the events it prints.
 */
 int	anni_adam_step_scaled(anni_adam *opt, double lr, double grad_scale);
 /* lm_adam_step. */
 int	anni_adam_step(anni_adam *opt, double lr);
+/*
+** lm_adam_set_offload (lm_adam.c:211-214) with adam_offload_mv (:314-334) and the re-upload of
+** gpu_buffers_init (:295-307): with on != 0 the moments leave the device after every step --
+** copied into two page-locked host buffers, their device blocks given back -- and the next step
+** (or checkpoint call) brings them back first; results do not change.  While they are away d_m
+** and d_v are NULL.  The first call with on != 0 moves m and v out of the arena's blocks into
+** blocks of their own (gpu_malloc) and everything else into new blocks without room for them, so
+** that the memory really is released: device pointers read from the handle before the call are
+** stale after it.  The moments leave at once, not only after the next step.  A step with the
+** moments offloaded allocates and waits, so it cannot be recorded into a HIP graph.  on == 0
+** brings the moments back and keeps them.  0 done, -1 failed (then nothing has moved).
+*/
+int	anni_adam_set_offload(anni_adam *opt, int on);
+/* 1 while m and v are on the device. */
+int	anni_adam_mv_on_device(const anni_adam *opt);
 /*
 ** Waits for the stream and fills last_sumsq / last_grad_norm / last_grad_scale / last_skipped /
 ** last_clipped; prints the reference's messages for that step on stderr (lm_adam.c:479-487):

@@ -1,8 +1,9 @@
 /*
-** anni_bench.h -- entry points of libanni_gpu_hip.so that exist for measuring and testing it:
-** event-timed step loops, synthetic input generators, a calibration copy kernel, re-reading of
-** the tuning switches.  Nothing a training program links against (that is anni_gpu.h and
-** anni_adam.h); bench.py and the tests call these.  None has a counterpart in the reference.
+** anni_bench.h -- libanni_bench.so: what measures and tests libanni_gpu_hip.so.  Event-timed
+** step loops, synthetic input generators, a calibration copy kernel, re-reading of the tuning
+** switches.  A library of its own, linked against libanni_gpu_hip.so: a training program links
+** only the latter (anni_gpu.h, anni_adam.h); bench.py and the tests load both.  None of these has
+** a counterpart in the reference.
 */
 #ifndef ANNI_BENCH_H__
 #define ANNI_BENCH_H__
@@ -41,6 +42,13 @@ int	anni_copy_bytes(void *d_dst, const void *d_src, size_t nbytes);
 ** depend on the switches.
 */
 void	anni_gpu_reload_switches(void);
+/*
+** The sum of squares checks its second stage against a conservative form of itself at its first
+** launch on a device and again after anni_gpu_reload_switches (two extra launches, one wait):
+** how often that check has run in this process and how often the two forms disagreed (then the
+** process has gone over to the conservative form and said so on stderr).  Returns 0.
+*/
+int	anni_fold_guard_stats(int *runs, int *mismatches);
 
 #ifdef __cplusplus
 }

@@ -297,6 +297,9 @@ def ref_hip():
 def _declare_model(R):
     R.ref_model_create.argtypes = [C.c_int, C.c_double, C.c_double, C.c_double]
     R.ref_model_create.restype = C.c_void_p
+    R.ref_model_create_tied.argtypes = [C.c_int, C.c_double, C.c_double, C.c_double]
+    R.ref_model_create_tied.restype = C.c_void_p
+    R.ref_model_dims.argtypes = [C.POINTER(C.c_int)] * 4
     R.ref_model_n.argtypes = [C.c_void_p]
     R.ref_model_n.restype = C.c_long
     for f in ("ref_model_n_segs", "ref_model_t", "ref_model_on_device"):
@@ -321,6 +324,25 @@ def _declare_model(R):
     R.ref_model_mv_on_device.argtypes = [C.c_void_p]
 
 
+# The same library compiled with the model sizes of the reference's 555M run
+# (scripts/run555m.sh:39-42: D=1536, 24 heads, FF=6272, 14 blocks).
+REF_HIP_555M_SO = os.path.join(HERE, "_ref", "libanni_ref_555m_hip.so")
+_ref_hip_555m = None
+
+
+def ref_hip_555m_available():
+    return os.path.exists(REF_HIP_555M_SO)
+
+
+def ref_hip_555m():
+    global _ref_hip_555m
+    if _ref_hip_555m is None:
+        R = C.CDLL(REF_HIP_555M_SO)
+        _declare_model(R)
+        _ref_hip_555m = R
+    return _ref_hip_555m
+
+
 _ref_cpu_model = None
 
 
@@ -337,13 +359,17 @@ def ref_cpu_model_lib():
 
 
 class RefModelOnBackend:
-    """The reference's real lm + lm_adam_create (its compile-time 185M sizes) on libanni_gpu_hip.so
-    (backend="hip") or on its own CPU stub (backend="cpu")."""
+    """The reference's real lm + lm_adam_create on libanni_gpu_hip.so, at its compile-time 185M
+    sizes (backend="hip") or at those of its 555M run (backend="hip555m"), or on its own CPU stub
+    (backend="cpu").  tied=True shares the head matrix with the embedding (lm_create_bpe_tied, what
+    `--tied` selects in the reference's training scripts)."""
 
     def __init__(self, vocab=16384, beta2=0.95, weight_decay=0.1, grad_clip=1.0, backend="hip",
-                 _handle=None):
-        self.R = ref_hip() if backend == "hip" else ref_cpu_model_lib()
-        self.h = _handle or self.R.ref_model_create(vocab, beta2, weight_decay, grad_clip)
+                 _handle=None, tied=False):
+        self.R = (ref_hip() if backend == "hip" else ref_hip_555m() if backend == "hip555m"
+                  else ref_cpu_model_lib())
+        create = self.R.ref_model_create_tied if tied else self.R.ref_model_create
+        self.h = _handle or create(vocab, beta2, weight_decay, grad_clip)
         if not self.h:
             raise MemoryError("ref_model_create")
         self.n = self.R.ref_model_n(self.h)
@@ -358,6 +384,12 @@ class RefModelOnBackend:
         if not h:
             raise ValueError("lm_load_checkpoint refused " + str(path))
         return cls(backend=backend, _handle=h), ep.value, st.value
+
+    def dims(self):
+        """(d_model, heads, d_ff, blocks) the library was compiled with."""
+        v = [C.c_int(0) for _ in range(4)]
+        self.R.ref_model_dims(*[C.byref(x) for x in v])
+        return tuple(x.value for x in v)
 
     def save_checkpoint(self, path, epoch, step):
         if self.R.ref_model_save_checkpoint(self.h, epoch, step, os.fsencode(path)) != 0:

@@ -17,6 +17,7 @@
 #include "train_progress.h"
 #include "layernorm.h"
 #include "lm_bench.h"
+#include "bpe.h"
 
 typedef struct ref_adam {
 	lm_adam	opt;
@@ -179,6 +180,72 @@ ref_model *ref_model_create(int vocab, double beta2, double wd, double clip)
 	r->opt->weight_decay = wd;
 	r->opt->grad_clip = clip;
 	return r;
+}
+
+/*
+** The same with the head matrix shared with the embedding, the way the reference trains its
+** larger models (`--tokenizer bpe --vocab V --tied`, scripts/run555m.sh:61-63): lm_create_bpe_tied
+** wants a tokenizer, so one with V - 260 synthetic merges is made (pairs of raw bytes first, then
+** byte + earlier merge: all distinct, every expansion at most three bytes); only its size matters
+** to the optimizer.  The model owns the tokenizer afterwards (lm_free releases it).
+*/
+ref_model *ref_model_create_tied(int vocab, double beta2, double wd, double clip)
+{
+	ref_model *r = calloc(1, sizeof(*r));
+	const int n_merges = vocab - BPE_BASE;
+	int *left = NULL;
+	int *right = NULL;
+	bpe *tok = NULL;
+	int i;
+
+	if (!r || n_merges < 0 || n_merges > 65536 * 2)
+		goto fail;
+	left = malloc((size_t)(n_merges ? n_merges : 1) * sizeof(int));
+	right = malloc((size_t)(n_merges ? n_merges : 1) * sizeof(int));
+	if (!left || !right)
+		goto fail;
+	for (i = 0; i < n_merges; i++) {
+		if (i < 65536) {
+			left[i] = VOCAB_SPECIALS + i / 256;
+			right[i] = VOCAB_SPECIALS + i % 256;
+		} else {
+			left[i] = VOCAB_SPECIALS + (i - 65536) % 256;
+			right[i] = BPE_BASE + (i - 65536) / 256;
+		}
+	}
+	tok = bpe_create(left, right, n_merges);
+	if (!tok)
+		goto fail;
+	r->model = lm_create_bpe_tied(tok);
+	if (!r->model) {
+		bpe_free(&tok);
+		goto fail;
+	}
+	r->opt = lm_adam_create(r->model);
+	if (!r->opt) {
+		lm_free(&r->model);
+		goto fail;
+	}
+	free(left);
+	free(right);
+	r->opt->beta2 = beta2;
+	r->opt->weight_decay = wd;
+	r->opt->grad_clip = clip;
+	return r;
+fail:
+	free(left);
+	free(right);
+	free(r);
+	return NULL;
+}
+
+/* The compile-time model sizes this library was built with (lang/lm_config.h:8-24). */
+void ref_model_dims(int *d_model, int *n_heads, int *d_ff, int *n_blocks)
+{
+	*d_model = LM_D_MODEL;
+	*n_heads = LM_N_HEADS;
+	*d_ff = LM_D_FF;
+	*n_blocks = LM_N_BLOCKS;
 }
 
 long ref_model_n(const ref_model *r) { return r->opt->n; }

@@ -14,25 +14,43 @@ from helpers import GOLDEN
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
+def declared_in(*headers):
     names = set()
-    for h in glob.glob(os.path.join(ROOT, "include", "*.h")):
+    for h in headers:
         text = open(h).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         names |= set(re.findall(r"\b((?:gpu|anni)_[a-z0-9_]+)\s*\(", text))
-    return sorted(names)
+    return names
 
 
-def test_every_declared_symbol_is_exported():
+def exported_by(so):
+    import subprocess
+    out = subprocess.check_output(["nm", "-D", "--defined-only", so]).decode()
+    return {ln.split()[-1] for ln in out.splitlines() if ln.strip()}
+
+
+def test_every_declared_symbol_is_exported_and_nothing_else():
+    """libanni_gpu_hip.so exports exactly what anni_gpu.h, anni_gpu_unserved.h and anni_adam.h
+    declare, plus the three hooks of the private header that libanni_bench.so is built on;
+    libanni_bench.so exports exactly what anni_bench.h declares.  No C++ symbol, no measuring or
+    testing utility in the product library."""
     from anni_amd import lib
-    L = C.CDLL(lib.SO_PATH)
-    syms = declared_symbols()
-    gpu = [s for s in syms if s.startswith("gpu_")]
-    assert len(gpu) == 99, len(gpu)          # the whole of num/gpu.h
-    for s in syms:
-        assert getattr(L, s) is not None, s
-    for s in lib._PROTOS:
-        assert s in syms, s
+    inc = os.path.join(ROOT, "include")
+    product = declared_in(os.path.join(inc, "anni_gpu.h"), os.path.join(inc, "anni_gpu_unserved.h"),
+                          os.path.join(inc, "anni_adam.h"))
+    hooks = declared_in(os.path.join(ROOT, "anni_amd", "csrc", "anni_hooks.h"))
+    bench = declared_in(os.path.join(inc, "anni_bench.h")) - product
+    assert len([s for s in product if s.startswith("gpu_")]) == 99          # the whole of num/gpu.h
+    assert hooks == {"anni_hook_step_events", "anni_hook_reload_switches", "anni_hook_fold_guard_stats"}
+    assert exported_by(lib.SO_PATH) == product | hooks
+    assert exported_by(lib.BENCH_SO_PATH) == bench
+    assert set(glob.glob(os.path.join(inc, "*.h"))) == {os.path.join(inc, h) for h in
+                                                        ("anni_gpu.h", "anni_gpu_unserved.h",
+                                                         "anni_adam.h", "anni_bench.h")}
+    for s_ in lib._PROTOS:
+        assert s_ in product, s_
+    for s_ in lib._BENCH_PROTOS:
+        assert s_ in bench, s_
 
 
 def test_missing_library_fails_loudly(monkeypatch):
@@ -187,3 +205,39 @@ def test_pool_chunk_bookkeeping_on_the_host(tmp_path):
                            os.path.join(ROOT, "tests", "c", "pool_chunks_test.cpp"), "-o", exe])
     out = subprocess.check_output([exe], timeout=120).decode()
     assert out.startswith("ok takes "), out
+
+
+def test_busy_flag_on_the_host(tmp_path):
+    """The flag that lets one gpu_grad_sumsq at a time at the shared result slot
+    (anni_amd/csrc/busy_flag.h) has no device call in it: eight threads, never two inside, a
+    caller that finds it taken is refused, the flag is free after every scope."""
+    import shutil
+    import subprocess
+    if not shutil.which("g++"):
+        pytest.skip("no g++")
+    exe = str(tmp_path / "busy_flag_test")
+    subprocess.check_call(["g++", "-std=c++17", "-O2", "-Wall", "-Wextra", "-Werror", "-pthread",
+                           "-I", os.path.join(ROOT, "anni_amd", "csrc"),
+                           os.path.join(ROOT, "tests", "c", "busy_flag_test.cpp"), "-o", exe])
+    out = subprocess.check_output([exe], timeout=120).decode()
+    assert out.startswith("ok entered "), out
+
+
+def test_division_by_a_step_constant_equals_the_ieee_quotient(tmp_path):
+    """div_by_const (anni_amd/csrc/adam_math.h: q = a * (1/b), one residual folded back, the sign
+    of a zero restored) restated on the host with fma() against a / b: b = 1 - beta^t for beta in
+    {0.9, 0.95, 0.999}, t = 1..10000, 3570 float-valued numerators each from every binary exponent
+    of a float, both signs, bf16-representable mantissas among them: 1.07e8 quotients, none may
+    differ.  (Without the sign fix every -0 numerator differed: -0 / b is -0, the residual form
+    gave +0.)"""
+    import shutil
+    import subprocess
+    if not shutil.which("gcc"):
+        pytest.skip("no gcc")
+    exe = str(tmp_path / "div_by_const_test")
+    subprocess.check_call(["gcc", "-O2", "-fopenmp", "-ffp-contract=off", "-Wall",
+                           os.path.join(ROOT, "tests", "c", "div_by_const_test.c"), "-o", exe, "-lm"])
+    out = subprocess.check_output([exe, "7"], timeout=600).decode().strip().splitlines()[-1]
+    words = out.split()
+    assert words[0] == "compared" and int(words[1]) >= 100000000, out
+    assert words[2] == "mismatches" and int(words[3]) == 0, out
