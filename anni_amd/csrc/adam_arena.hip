@@ -65,6 +65,7 @@ struct anni_adam_priv {
 	int			logged_t;	/* the step whose messages anni_adam_sync_stats has printed */
 	int			split;		/* 1: two allocations (see the layout note in anni_adam_create) */
 	double			probe_gbps;	/* update throughput measured at creation (0: not measured) */
+	PlaceStats		search;		/* split: what the search for the second block cost */
 	std::vector<int64_t>	offsets;
 	std::vector<uint32_t>	flags;
 	/* derived outputs (anni_adam_enable_derived): one more allocation */
@@ -97,6 +98,7 @@ struct Placement {
 	int	split;
 	double	ratio;		/* split: what alloc_apart_from measured */
 	double	gbps;		/* what the full-size probe measured (0: not probed) */
+	PlaceStats	search;	/* split: what the search for the second block cost */
 };
 
 /*
@@ -151,7 +153,7 @@ static bool place(const Sizes &z, bool split, Placement *pl)
 	pl->a = (char *)mem;
 	if (split) {
 		/* p and m are still scratch: the search times the update on them and on each candidate */
-		pl->b = (char *)alloc_apart_from(pl->a, pl->off_gscale, pl->b_bytes, &pl->ratio);
+		pl->b = (char *)alloc_apart_from(pl->a, pl->off_gscale, pl->b_bytes, &pl->ratio, &pl->search);
 		if (!pl->b) {
 			(void)hipFree(pl->a);
 			pl->a = nullptr;
@@ -186,6 +188,7 @@ static void adopt(anni_adam *opt, const Sizes &z, const Placement &pl)
 	pv->split = pl.split;
 	pv->apart_ratio = pl.ratio;
 	pv->probe_gbps = pl.gbps;
+	pv->search = pl.search;
 	opt->d_param = (float *)(base + pl.off_p);
 	opt->d_m = base + pl.off_m;
 	opt->d_v = second + pl.off_v;
@@ -528,6 +531,17 @@ double anni_adam_probe_gbps(const anni_adam *opt)
 	return opt && opt->priv ? opt->priv->probe_gbps : 0.0;
 }
 
+int anni_adam_placement_cost(const anni_adam *opt, double *walked_gib, double *ms)
+{
+	if (!opt || !opt->priv)
+		return -1;
+	if (walked_gib)
+		*walked_gib = opt->priv->search.walked_gib;
+	if (ms)
+		*ms = opt->priv->search.ms;
+	return opt->priv->search.timed;
+}
+
 static void describe(const anni_adam *opt, Flat *f);
 
 /* The derived outputs as the update would leave them, straight from p. */
@@ -614,8 +628,7 @@ static int enable_derived_body(anni_adam *opt, const anni_pack *packs, int n_pac
 	off_pack = round_up(off_tamax + (fp8 ? (size_t)((opt->n + kTile - 1) / kTile) * kWaves
 	    * sizeof(float) : 0), (size_t)2 << 20);
 	total = off_pack + round_up((size_t)pack_elems * 2, 256) + 256;
-	if (hipMalloc(&pv->derived, total) != hipSuccess) {
-		(void)hipGetLastError();
+	if (device_alloc(&pv->derived, total) != hipSuccess) {
 		pv->derived = nullptr;
 		return -1;
 	} else {
@@ -710,11 +723,9 @@ int anni_adam_quantize_grads(anni_adam *opt, const float *d_src)
 		const size_t amax_bytes = round_up((size_t)opt->n_tensors * sizeof(uint32_t), 256);
 		void *d = nullptr;
 
-		if (!hip_ok(hipMalloc(&d, amax_bytes + n_tiles * kWaves * sizeof(float)),
-		    "quantizer hipMalloc")) {
-			(void)hipGetLastError();
+		if (!hip_ok(device_alloc(&d, amax_bytes + n_tiles * kWaves * sizeof(float)),
+		    "quantizer hipMalloc"))
 			return -1;
-		}
 		pv->gq_scratch = d;
 	}
 	return quantize_grads_into(opt, d_src, pv->gq_scratch);
@@ -1184,7 +1195,7 @@ struct CkptStage {
 
 		for (int i = 0; i < 2; i++) {
 			if (hipHostMalloc((void **)&host[i], bytes, hipHostMallocDefault) != hipSuccess
-			    || hipMalloc((void **)&dev[i], bytes) != hipSuccess
+			    || device_alloc((void **)&dev[i], bytes) != hipSuccess
 			    || hipEventCreateWithFlags(&ev[i], hipEventDisableTiming) != hipSuccess) {
 				(void)hipGetLastError();
 				return false;

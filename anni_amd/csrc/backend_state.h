@@ -29,6 +29,12 @@ bool		hip_ok(hipError_t err, const char *what);
 ** large reservations.
 */
 bool		release_idle_pools(void);
+/*
+** hipMalloc for the library's own blocks (scratch, derived outputs, staging): when the driver
+** has nothing left, the empty chunks of gpu_malloc's pools are given back and the request is
+** made once more.  *p is NULL on failure; the error is cleared.
+*/
+hipError_t	device_alloc(void **p, size_t nbytes);
 
 /*
 ** ANN_OP_PROF=1 (num/gpu_cuda.cu:3205-3409): an event pair around an operation of the optimizer

@@ -475,7 +475,7 @@ int gpu_mem_info(size_t *free_bytes, size_t *total_bytes)
 	{
 		std::lock_guard<std::mutex> lk(g_pool_mu);
 
-		f += pools_idle_bytes_locked();	/* reserved, but given back on demand */
+		f += pools_idle_bytes_locked();	/* reserved, but there for the asking */
 	}
 	if (free_bytes)
 		*free_bytes = f;
@@ -615,42 +615,90 @@ static char *pool_scratch(int pool, size_t *bytes)
 	return best;
 }
 
-/* g_pool_mu held.  A block of a pool, or nullptr (the caller then allocates the plain way). */
+static bool g_pool_growing;		/* one thread at a time looks for a new chunk */
+
+/*
+** A block of a pool, or nullptr (the caller then allocates the plain way).  Takes g_pool_mu
+** itself and lets go of it while it looks for a new chunk: the search requests and times tens of
+** GiB and takes tens of milliseconds, and every other thread's gpu_malloc, gpu_free and
+** gpu_mem_info would wait that long.  What the search needs from the pools -- the free space of
+** the other pool that it uses as scratch -- is reserved as a block for the time, so nobody is
+** handed it and its chunk does not count as idle; a second thread that needs a new chunk
+** meanwhile gets a plain allocation.
+*/
 static void *pool_take(size_t nbytes)
 {
 	const size_t need = (nbytes + ((size_t)2 << 20) - 1) & ~(((size_t)2 << 20) - 1);
-	const int pool = g_pool_live[1] < g_pool_live[0] ? 1 : 0;
 	size_t fr = 0, tt = 0, scratch_bytes = 0;
 	size_t chunk_bytes = 4 * need;
-	char *scratch;
+	PoolChunk *scratch_chunk = nullptr;
+	char *scratch = nullptr;
 	void *mem = nullptr;
+	void *got = nullptr;
+	int pool;
 
-	for (PoolChunk &have : g_chunks)
-		if (have.pool == pool) {
-			void *p = chunk_take(have, need);
+	{
+		std::lock_guard<std::mutex> lk(g_pool_mu);
 
-			if (p)
-				return p;
+		pool = g_pool_live[1] < g_pool_live[0] ? 1 : 0;
+		for (PoolChunk &have : g_chunks)
+			if (have.pool == pool) {
+				void *p = chunk_take(have, need);
+
+				if (p)
+					return p;
+			}
+		if (g_pool_growing)
+			return nullptr;
+		if (hipMemGetInfo(&fr, &tt) != hipSuccess) {
+			(void)hipGetLastError();
+			return nullptr;
 		}
-	if (hipMemGetInfo(&fr, &tt) != hipSuccess) {
-		(void)hipGetLastError();
-		return nullptr;
+		if (chunk_bytes > fr / 8)
+			chunk_bytes = need;		/* memory is short: no more than what is asked for */
+		if (chunk_bytes > fr / 2)
+			return nullptr;
+		scratch = pool_scratch(1 - pool, &scratch_bytes);
+		if (scratch) {
+			for (PoolChunk &c : g_chunks)
+				if (scratch >= c.base && scratch < c.base + c.bytes)
+					scratch_chunk = &c;
+			if (!scratch_chunk || scratch_chunk->take_block((size_t)(scratch - scratch_chunk->base))
+			    != scratch_bytes)
+				return nullptr;
+		}
+		g_pool_growing = true;
 	}
-	if (chunk_bytes > fr / 8)
-		chunk_bytes = need;		/* memory is short: no more than what is asked for */
-	if (chunk_bytes > fr / 2)
-		return nullptr;
-	scratch = pool_scratch(1 - pool, &scratch_bytes);
-	if (scratch) {
-		mem = alloc_apart_from(scratch, scratch_bytes, chunk_bytes, nullptr);
-	} else if (hipMalloc(&mem, chunk_bytes) != hipSuccess) {
-		(void)hipGetLastError();
-		mem = nullptr;
+	/* the lock is free; g_chunks may grow or shrink meanwhile, so the reservation is found again by address */
+	try {
+		if (scratch) {
+			mem = alloc_apart_from(scratch, scratch_bytes, chunk_bytes, nullptr);
+		} else if (hipMalloc(&mem, chunk_bytes) != hipSuccess) {
+			(void)hipGetLastError();
+			mem = nullptr;
+		}
+	} catch (...) {
+		mem = nullptr;		/* the reservation and the flag below are undone all the same */
 	}
-	if (!mem)
-		return nullptr;
-	g_chunks.push_back(PoolChunk((char *)mem, chunk_bytes, pool));
-	return chunk_take(g_chunks.back(), need);
+	{
+		std::lock_guard<std::mutex> lk(g_pool_mu);
+
+		g_pool_growing = false;
+		if (scratch)
+			for (PoolChunk &c : g_chunks)
+				if (scratch >= c.base && scratch < c.base + c.bytes)
+					(void)c.give((size_t)(scratch - c.base));
+		if (mem) {
+			try {
+				g_chunks.push_back(PoolChunk((char *)mem, chunk_bytes, pool));
+				got = chunk_take(g_chunks.back(), need);
+			} catch (...) {
+				(void)hipFree(mem);
+				got = nullptr;
+			}
+		}
+	}
+	return got;
 }
 
 /*
@@ -673,14 +721,17 @@ static int pool_give(void *p)
 	return 0;
 }
 
-/* g_pool_mu held.  Bytes of chunks that are reserved but hold no block. */
+/*
+** g_pool_mu held.  Bytes the pools hold without a block in them: whole chunks that are empty
+** (given back to the driver on demand) and the free space inside chunks that are in use (handed
+** out by the next large gpu_malloc).
+*/
 static size_t pools_idle_bytes_locked(void)
 {
 	size_t idle = 0;
 
 	for (const PoolChunk &c : g_chunks)
-		if (c.live == 0)
-			idle += c.bytes;
+		idle += c.bytes - c.live;
 	return idle;
 }
 
@@ -712,8 +763,6 @@ void *gpu_malloc(size_t nbytes)
 	if (nbytes >= kPlaceMin && place_on()) {
 		batch_flush();			/* the placement probe runs on the compute stream */
 		try {
-			std::lock_guard<std::mutex> lk(g_pool_mu);
-
 			p = pool_take(nbytes);
 		} catch (...) {
 			p = nullptr;
@@ -927,10 +976,8 @@ static void twin_check(const void *twin, const ann_real *fp32, size_t n)
 	unsigned char *a, *b;
 	size_t bad = 0;
 
-	if (hipMalloc(&fresh, bytes) != hipSuccess) {
-		(void)hipGetLastError();
+	if (device_alloc(&fresh, bytes) != hipSuccess)
 		return;
-	}
 	a = (unsigned char *)malloc(bytes);
 	b = (unsigned char *)malloc(bytes);
 	if (a && b && launch_f32_to_bf16(stream_for_op(), (uint16_t *)fresh, fp32, (int64_t)n) == 0
@@ -1076,6 +1123,21 @@ bool release_idle_pools(void)
 	std::lock_guard<std::mutex> lk(g_pool_mu);
 
 	return pools_release_idle_locked();
+}
+
+hipError_t device_alloc(void **p, size_t nbytes)
+{
+	hipError_t err = hipMalloc(p, nbytes);
+
+	if (err != hipSuccess && release_idle_pools()) {
+		(void)hipGetLastError();
+		err = hipMalloc(p, nbytes);
+	}
+	if (err != hipSuccess) {
+		(void)hipGetLastError();
+		*p = nullptr;
+	}
+	return err;
 }
 
 } /* namespace anni */

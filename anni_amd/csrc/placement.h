@@ -26,20 +26,32 @@ namespace anni {
 /* Blocks smaller than this are not worth placing (their streams are short). */
 constexpr size_t kPlaceMin = (size_t)256 << 20;
 
+/* What a search did, for the record (anni_adam_placement_stats, ANNI_PLACE_LOG=1). */
+struct PlaceStats {
+	double	walked_gib;	/* device memory requested and held during the walk, the result included */
+	double	ms;		/* wall clock of the whole search */
+	int	timed;		/* candidates that were timed */
+};
+
 /*
 ** Allocates `bytes` of device memory that streams well together with the block
 ** [ref, ref + ref_bytes): memory of another section when one can be had.  Blocks of `bytes` are
 ** requested one after the other and kept (the allocator works its way down through the
 ** sections), about every 8 GiB one of them is timed against `ref`, until one is at least 7 %
-** faster than the same launch inside a single block, 200 GiB have been walked (ANNI_PLACE_MAX_GIB
-** sets another limit) or memory runs low; the best one is kept, all others are returned.  Both probe areas -- the first 18 bytes per probe element of `ref` and of
-** every candidate -- are zero-filled and left zero, so `ref` must not hold data there.  *ratio
-** (may be NULL) receives time(one block) / time(ref + result), "one block" being the slower of
-** `ref` alone and the first candidate alone; 1.0 when nothing was measured.  A ratio near 1 with
-** a fast arena happens too: memory the driver reuses after frees is often pieced together from
-** several sections already, and then there is nothing left to gain.  NULL when the allocation itself fails.  Synchronises the compute stream.
+** faster than the same launch inside a single block or the walk has reached its limit; the best
+** one is kept, all others are returned.  The limit: one section and one block (96 GiB + `bytes`;
+** ANNI_PLACE_MAX_GIB sets another figure, 0 = no walk), and never more than half of what was
+** free when the search began, so that the process and its neighbours on the device keep room
+** to allocate while it runs.  Both probe areas -- the first 18 bytes per probe element of `ref`
+** and of every candidate -- are zero-filled and left zero, so `ref` must not hold data there.
+** *ratio (may be NULL) receives time(one block) / time(ref + result), "one block" being the
+** slower of `ref` alone and the first candidate alone; 1.0 when nothing was measured.  A ratio
+** near 1 with a fast arena happens too: memory the driver reuses after frees is often pieced
+** together from several sections already, and then there is nothing left to gain.  NULL when the
+** allocation itself fails.  Synchronises the compute stream.  Takes no lock of this library.
 */
-void	*alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio);
+void	*alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio,
+		PlaceStats *stats = nullptr);
 
 } /* namespace anni */
 #endif

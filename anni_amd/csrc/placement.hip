@@ -6,6 +6,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <chrono>
 #include <vector>
 #include "adam_kernels.h"
 #include "backend_state.h"
@@ -16,7 +17,7 @@ namespace anni {
 static const int64_t kProbeElems = (int64_t)64 << 20;	/* 0.34 ms per launch; shorter launches tell less */
 static const int64_t kProbeMinElems = (int64_t)8 << 20;
 static const size_t kProbeEvery = (size_t)8 << 30;	/* a block is timed about every 8 GiB of blocks */
-static const size_t kWalkMax = (size_t)200 << 30;	/* a section is 96 GiB: two of them, and some for gaps */
+static const size_t kSection = (size_t)96 << 30;	/* the walk crosses a section boundary within one section's worth of blocks */
 static const double kApartRatio = 1.07;			/* measured 1.13 - 1.17 across a section boundary */
 
 /*
@@ -89,19 +90,22 @@ static bool place_log(void)
 	return on == 1;
 }
 
-/* How far the walk may go: ANNI_PLACE_MAX_GIB (default 200; 0 = no walk, the first block is taken). */
-static size_t walk_max(void)
+/*
+** How far the walk may go: one section and one block, or ANNI_PLACE_MAX_GIB GiB when that is set
+** (0 = no walk, the first block is taken).
+*/
+static size_t walk_max(size_t bytes)
 {
-	static long gib = -1;
+	static long gib = -2;
 
-	if (gib < 0) {
+	if (gib == -2) {
 		const char *e = getenv("ANNI_PLACE_MAX_GIB");
 
-		gib = e && *e ? atol(e) : (long)(kWalkMax >> 30);
-		if (gib < 0 || gib > 1024)
-			gib = (long)(kWalkMax >> 30);
+		gib = e && *e ? atol(e) : -1;
+		if (gib < -1 || gib > 1024)
+			gib = -1;
 	}
-	return (size_t)gib << 30;
+	return gib >= 0 ? (size_t)gib << 30 : kSection + bytes;
 }
 
 static size_t free_bytes_now(size_t *total)
@@ -118,12 +122,14 @@ static size_t free_bytes_now(size_t *total)
 	return fr;
 }
 
-void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio)
+void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio, PlaceStats *stats)
 {
 	hipStream_t st = compute_stream();
+	const auto t_begin = std::chrono::steady_clock::now();
 	std::vector<void *> blocks;
 	size_t walked = 0;
 	size_t total = 0;
+	int timed = 0;
 	double t_same = 0.0;
 	double best_ratio = 0.0;
 	int best = -1;
@@ -131,6 +137,8 @@ void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio)
 
 	if (ratio)
 		*ratio = 1.0;
+	if (stats)
+		memset(stats, 0, sizeof(*stats));
 	/* probe size: 18 bytes per element inside ref and inside a candidate (for the one-block timings) */
 	n = kProbeElems;
 	if ((size_t)n * 18 > ref_bytes)
@@ -145,10 +153,14 @@ void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio)
 			(void)hipGetLastError();
 			return nullptr;
 		}
+		if (stats)
+			stats->walked_gib = (double)bytes / 1073741824.0;
 		return p;
 	}
-	(void)free_bytes_now(&total);
+	const size_t free_at_entry = free_bytes_now(&total);
 	const size_t margin = total / 20 > ((size_t)8 << 30) ? total / 20 : ((size_t)8 << 30);
+	/* never more than half of what is free now: others allocate while this runs */
+	const size_t limit = walk_max(bytes) < free_at_entry / 2 ? walk_max(bytes) : free_at_entry / 2;
 	/*
 	** The walk: blocks of `bytes` are requested one after the other and kept, so the allocator
 	** works its way down through device memory; about every 8 GiB one of them is timed.  The
@@ -162,7 +174,7 @@ void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio)
 
 	if (launch_fill_bytes(st, ref, 0, (size_t)n * 18) != 0)
 		return nullptr;
-	for (size_t it = 0; it == 0 || walked < walk_max(); it++) {
+	for (size_t it = 0; it == 0 || walked + bytes <= limit; it++) {
 		void *c = nullptr;
 		double t_pair;
 
@@ -195,6 +207,7 @@ void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio)
 		t_pair = probe_ms((char *)ref, (char *)c, n);
 		if (t_pair <= 0.0)
 			break;
+		timed++;
 		if (place_log())
 			fprintf(stderr, "[place] block %zu at %p (%.2f GiB): one block %.4f ms, with ref %p %.4f ms, "
 			    "ratio %.3f, walked %.0f GiB, free %.1f GiB\n", it, c, (double)bytes / 1073741824.0,
@@ -214,6 +227,17 @@ void *alloc_apart_from(void *ref, size_t ref_bytes, size_t bytes, double *ratio)
 		if ((int)i != best)
 			(void)hipFree(blocks[i]);
 	(void)hipGetLastError();
+	if (stats) {
+		stats->walked_gib = (double)walked / 1073741824.0;
+		stats->ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now()
+		    - t_begin).count();
+		stats->timed = timed;
+	}
+	if (place_log())
+		fprintf(stderr, "[place] search over: %.1f GiB walked in %zu blocks, %d timed, %.1f ms, best ratio %.3f\n",
+		    (double)walked / 1073741824.0, blocks.size(), timed,
+		    std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t_begin).count(),
+		    best_ratio);
 	if (best < 0)
 		return nullptr;
 	if (ratio && best_ratio > 0.0)

@@ -49,6 +49,22 @@ struct PoolChunk {
 		return (size_t)-1;
 	}
 
+	/*
+	** Takes the whole free block that starts at `off` (what largest_free reported): its size, or
+	** 0 when no free block starts there.  For a reservation that is handed back with give().
+	*/
+	size_t take_block(size_t off)
+	{
+		for (size_t i = 0; i < blocks.size(); i++) {
+			if (blocks[i].off != off || blocks[i].used)
+				continue;
+			blocks[i].used = true;
+			live += blocks[i].bytes;
+			return blocks[i].bytes;
+		}
+		return 0;
+	}
+
 	/* Bytes given back by freeing the live block that starts at `off`; 0 when there is none. */
 	size_t give(size_t off)
 	{

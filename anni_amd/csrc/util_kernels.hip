@@ -353,7 +353,7 @@ int gpu_mat_col_sum_add(ann_real *db_host, const ann_real *x, int rows, int cols
 	if (cols > d_acc_cols) {
 		void *p = nullptr;
 
-		if (!hip_ok(hipMalloc(&p, (size_t)cols * sizeof(float)), "colsum hipMalloc")) {
+		if (!hip_ok(device_alloc(&p, (size_t)cols * sizeof(float)), "colsum hipMalloc")) {
 			(void)hipGetLastError();
 			return -1;
 		}

@@ -98,6 +98,7 @@ _PROTOS = {
     "anni_adam_is_split": (C.c_int, [C.POINTER(Adam)]),
     "anni_adam_apart_ratio": (C.c_double, [C.POINTER(Adam)]),
     "anni_adam_probe_gbps": (C.c_double, [C.POINTER(Adam)]),
+    "anni_adam_placement_cost": (C.c_int, [C.POINTER(Adam), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "anni_adam_arena_bytes": (C.c_size_t, [C.POINTER(Adam)]),
     "anni_adam_resident_bytes": (C.c_size_t, [C.POINTER(Adam)]),
     "anni_adam_bind_grad": (C.c_int, [C.POINTER(Adam), C.c_void_p]),

@@ -110,60 +110,143 @@ def fill_grad_slots(L, opt, tensors, count, grad_type, seed, first_step=0):
 
 def short_leg(L, workload, layout, steps=6, warmup=2, slots=4):
     """A second arena in the same process (after the first was freed): `steps` timed steps of
-    `workload` on an arena of the given layout, HIP events per kernel.  For the all-f32 workloads."""
+    `workload` on an arena of the given layout, HIP events per kernel, any storage mode."""
     from anni_amd import layout as lay
     from anni_amd import lm_adam
     from anni_amd.lm_adam import LmAdam
     size, gt, mt, norm_bpp, upd_bpp = WORKLOADS[workload]
-    assert gt == 0 and mt == 0
     tensors = lay.tensors(size, "baseline")
-    opt = LmAdam(tensors, twins=True, skip_nonfinite=True, grad_slots=slots,
+    t_create = time.perf_counter()
+    opt = LmAdam(tensors, grad_type=gt, moment_type=mt, twins=True, skip_nonfinite=True, grad_slots=slots,
                  layout={"auto": 0, "compact": 1, "split": 2}[layout],
                  beta2=0.95, weight_decay=0.1, grad_clip=1.0)
+    t_create = (time.perf_counter() - t_create) * 1e3
     n = opt.n
+    own_gscale = opt.o.d_gscale
     assert L.anni_fill_normal_f32(opt.o.d_param, n, 20260101, 1, 0.0, 0.02) == 0
     opt.seed_twins()
     unit = 1.0 / (math.sqrt(n) * 1e-3)
     tot = [0.0, 0.0, 0.0]
     wall = 0.0
     done = 0
+    old_scales = []
     while done < warmup + steps:
         count = min(slots, warmup + steps - done)
-        ring, _sc = fill_grad_slots(L, opt, tensors, count, 0, 20260101, done)
-        ptrs = (C.c_void_p * count)(*ring)
-        lr = (C.c_double * count)(*[lm_adam.step_lr(3e-4, done + i, 100, 1000, "cosine") for i in range(count)])
-        gs = (C.c_double * count)(*[unit * (1.7 if (done + i) % 2 else 0.6) for i in range(count)])
+        ring, scales = fill_grad_slots(L, opt, tensors, count, gt, 20260101, done)
+        for sc in old_scales:
+            if sc is not None:
+                sc.free()
+        old_scales = scales
+        lr = [lm_adam.step_lr(3e-4, done + i, 100, 1000, "cosine") for i in range(count)]
+        gs = [unit * (1.7 if (done + i) % 2 else 0.6) for i in range(count)]
         timed = [i for i in range(count) if done + i >= warmup]
-        if len(timed) < count:                           # the warm-up part of this batch
-            k = count - len(timed)
-            ms = C.c_float(0)
-            assert L.anni_adam_time_steps(opt.h, k, ptrs, k, lr, gs, C.byref(ms), None, None) == 0
-        if timed:
-            k0, k = timed[0], len(timed)
+
+        def run(first, k, per_kernel):
+            """Steps first .. first + k - 1 of this batch; fp8: one call per step, each flat has scales of its own."""
             ms, sa, sb = C.c_float(0), C.c_float(0), C.c_float(0)
-            sub = (C.c_void_p * k)(*ring[k0:])
+            groups = [(first + i, 1) for i in range(k)] if gt == 2 else [(first, k)]
+            out = [0.0, 0.0, 0.0]
+            for g0, gk in groups:
+                if gt == 2:
+                    opt.o.d_gscale = scales[g0].ptr
+                rc = L.anni_adam_time_steps(opt.h, gk, (C.c_void_p * gk)(*ring[g0:g0 + gk]), gk,
+                                            (C.c_double * gk)(*lr[g0:g0 + gk]),
+                                            (C.c_double * gk)(*gs[g0:g0 + gk]), C.byref(ms),
+                                            C.byref(sa) if per_kernel else None,
+                                            C.byref(sb) if per_kernel else None)
+                assert rc == 0, L.gpu_debug_last_error()
+                out = [out[0] + ms.value, out[1] + sa.value, out[2] + sb.value]
+            return out
+        if len(timed) < count:                           # the warm-up part of this batch
+            run(0, count - len(timed), False)
+        if timed:
             L.gpu_device_sync()
             t0 = time.perf_counter()
-            assert L.anni_adam_time_steps(opt.h, k, sub, k, (C.c_double * k)(*lr[k0:]),
-                                          (C.c_double * k)(*gs[k0:]), C.byref(ms), C.byref(sa),
-                                          C.byref(sb)) == 0, L.gpu_debug_last_error()
+            got = run(timed[0], len(timed), True)
             L.gpu_device_sync()
             wall += (time.perf_counter() - t0) * 1e3
-            tot = [tot[0] + ms.value, tot[1] + sa.value, tot[2] + sb.value]
+            tot = [tot[0] + got[0], tot[1] + got[1], tot[2] + got[2]]
         done += count
     st = opt.sync_stats()
     assert opt.t == warmup + steps and math.isfinite(st.last_grad_norm)
-    ms_step, upd_ms = wall / steps, tot[2] / steps
-    out = {"workload": workload, "params": n, "steps": steps, "warmup": warmup,
+    # fp8: a step per call, so the wall clock carries a launch and a wait per step; the events do not
+    ms_step = (tot[0] if gt == 2 else wall) / steps
+    upd_ms = tot[2] / steps
+    walked, place_ms, _timed = opt.placement_cost
+    _traffic, _digest, current = profiled_traffic(workload)
+    out = {"workload": workload, "storage": STORAGE[workload], "params": n, "steps": steps, "warmup": warmup,
            "layout": "split" if opt.split else "compact",
            "placement_apart_ratio": round(opt.apart_ratio, 3),
+           "placement_walked_GiB": round(walked, 1), "placement_ms": round(place_ms, 1),
+           "arena_create_ms": round(t_create, 1),
            "arena_bytes": opt.arena_bytes, "resident_bytes": opt.resident_bytes,
            "ms_per_step": round(ms_step, 4),
+           "ms_per_step_timed_by": "events around each step" if gt == 2 else "wall clock around the run",
            "GBps": round(n * (norm_bpp + upd_bpp) / ms_step / 1e6, 1),
            "frac": round(n * (norm_bpp + upd_bpp) / ms_step / 1e6 / HBM_PEAK_GBPS, 4),
            "update_ms": round(upd_ms, 4), "sumsq_ms": round(tot[1] / steps, 4),
-           "update_frac": round(n * upd_bpp / upd_ms / 1e6 / HBM_PEAK_GBPS, 4)}
+           "update_frac": round(n * upd_bpp / upd_ms / 1e6 / HBM_PEAK_GBPS, 4),
+           "profile_matches_these_sources": current}
+    opt.o.d_gscale = own_gscale
+    for sc in old_scales:
+        if sc is not None:
+            sc.free()
     opt.free()
+    return out
+
+
+def placement_cost_leg(L):
+    """What the search for the arena's second block costs, and what it leaves behind for the next
+    allocation: creation of a 555M arena (GiB requested and held during the walk, milliseconds),
+    then hipMalloc + first touch of 64 GiB; first on the device as this process found it, then again
+    after 150 GiB were allocated, touched and freed.  Run with ANNI_PLACE_LOG=1 to see every candidate."""
+    from anni_amd import layout as lay
+    from anni_amd.lm_adam import LmAdam
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+    hip.hipFree.argtypes = [C.c_void_p]
+    tensors = lay.tensors("555m", "baseline")
+
+    def malloc_and_touch(gib):
+        p = C.c_void_p()
+        L.gpu_device_sync()
+        t0 = time.perf_counter()
+        assert hip.hipMalloc(C.byref(p), gib << 30) == 0
+        t1 = time.perf_counter()
+        assert L.gpu_memset(p.value, 0, gib << 30) == 0
+        L.gpu_device_sync()
+        t2 = time.perf_counter()
+        assert hip.hipFree(p) == 0
+        L.gpu_device_sync()
+        return {"GiB": gib, "hipMalloc_ms": round((t1 - t0) * 1e3, 1), "first_fill_ms": round((t2 - t1) * 1e3, 1),
+                "hipFree_ms": round((time.perf_counter() - t2) * 1e3, 1)}
+
+    def create():
+        fr, tt = C.c_size_t(0), C.c_size_t(0)
+        L.gpu_mem_info(C.byref(fr), C.byref(tt))
+        t0 = time.perf_counter()
+        opt = LmAdam(tensors, twins=True, skip_nonfinite=True, grad_slots=13, beta2=0.95,
+                     weight_decay=0.1, grad_clip=1.0)
+        ms = (time.perf_counter() - t0) * 1e3
+        walked, place_ms, timed = opt.placement_cost
+        out = {"free_GiB_before": round(fr.value / (1 << 30), 1), "create_ms": round(ms, 1),
+               "search_ms": round(place_ms, 1), "walked_GiB": round(walked, 1), "candidates_timed": timed,
+               "apart_ratio": round(opt.apart_ratio, 3), "probe_GBps": round(opt.probe_gbps, 1),
+               "arena_GiB": round(opt.arena_bytes / (1 << 30), 2)}
+        opt.free()
+        return out
+    out = {"untouched_device": {"arena_create": create(), "then_64GiB": malloc_and_touch(64),
+                                "64GiB_again": malloc_and_touch(64)}}
+    blocks = []
+    for _ in range(150 // 15):
+        p = C.c_void_p()
+        assert hip.hipMalloc(C.byref(p), 15 << 30) == 0
+        assert L.gpu_memset(p.value, 1, 15 << 30) == 0
+        blocks.append(p)
+    L.gpu_device_sync()
+    for p in blocks:
+        assert hip.hipFree(p) == 0
+    out["after_150GiB_allocated_touched_freed"] = {"arena_create": create(), "then_64GiB": malloc_and_touch(64)}
     return out
 
 
@@ -558,6 +641,8 @@ def main():
                          "flats in chosen blocks: shows the three 96 GiB sections the placement is about")
     ap.add_argument("--colsum", type=int, default=0, metavar="ROWS",
                     help="only time the bias / LayerNorm gradient column sums over ROWS token rows")
+    ap.add_argument("--placement-cost", action="store_true",
+                    help="only measure what the search for the arena's second block costs and leaves behind")
     ap.add_argument("--reference-caller-only", action="store_true",
                     help="only time the unchanged reference caller on this backend (one JSON line)")
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds for the CPU legs")
@@ -598,6 +683,9 @@ def main():
         return
     if a.colsum:
         print(json.dumps({"colsum_add": colsum_leg(L, a.colsum)}))
+        return
+    if a.placement_cost:
+        print(json.dumps({"placement_cost": placement_cost_leg(L)}))
         return
     if a.reference_caller_only:
         print(json.dumps({"reference_caller_185m": reference_caller_leg(L, "185m"),
@@ -733,6 +821,8 @@ def main():
                    "layout": "split" if opt.split else "compact",
                    "placement_apart_ratio": round(opt.apart_ratio, 3),
                    "placement_probe_GBps": round(opt.probe_gbps, 1),
+                   "placement_walked_GiB": round(opt.placement_cost[0], 1),
+                   "placement_ms": round(opt.placement_cost[1], 1),
                    "arena_bytes": opt.arena_bytes, "resident_bytes": opt.resident_bytes,
                    "grad_slots": n_slots, "arena_create_ms": round(t_create, 1),
                    "launches_per_step": 2},
@@ -786,7 +876,9 @@ def main():
         # metric names, each on an arena of its own after the headline's was freed
         try:
             out["layout_compact"] = short_leg(L, "555m", "compact")
-            out["workloads"] = {"185m": short_leg(L, "185m", "auto")}
+            out["workloads"] = {}
+            for w in ("185m", "555m-bf16", "1p4b-fp8"):
+                out["workloads"][w] = short_leg(L, w, "auto")
         except Exception as e:                      # a side leg must never sink the bench line
             out["side_legs_error"] = repr(e)
     if not a.no_cpu:

@@ -44,9 +44,10 @@ extern "C" {
 ** contents -- p, m and the tables in one; v, the twins and the gradient slots in the other -- and
 ** looks for the second in another section by timing the update on the (still empty) flats:
 ** blocks of its size are requested one after the other and kept, every 8 GiB one is timed, until
-** one is fast, 200 GiB have been walked or memory runs low, and everything but the arena is
-** returned before anni_adam_create returns (for a moment up to ~200 GiB more than the arena are
-** held; with little memory free the search just ends sooner).
+** one is fast or the walk has covered one section and one block (96 GiB + the block), never more
+** than half of what was free when it began; everything but the arena is returned before
+** anni_adam_create returns (anni_adam_placement_cost says what was held and for how long;
+** ANNI_PLACE_MAX_GIB sets another limit, 0 = no search).
 ** COMPACT is one allocation.  AUTO splits when the parameter flat has 256 MiB or more.
 */
 #define ANNI_LAYOUT_AUTO	0
@@ -143,6 +144,13 @@ int	anni_adam_is_split(const anni_adam *opt);
 */
 double	anni_adam_apart_ratio(const anni_adam *opt);
 double	anni_adam_probe_gbps(const anni_adam *opt);
+/*
+** What the search for the second block cost at creation: GiB of device memory requested and held
+** while it ran (the block that was kept included) and its wall-clock time; returns the number of
+** candidate blocks that were timed (0 for a compact arena or when nothing was searched), -1 for
+** a bad handle.
+*/
+int	anni_adam_placement_cost(const anni_adam *opt, double *walked_gib, double *ms);
 /* Device memory the arena holds, and what one step touches (p, m, v, twins, one gradient flat, tables). */
 size_t	anni_adam_arena_bytes(const anni_adam *opt);
 size_t	anni_adam_resident_bytes(const anni_adam *opt);

@@ -124,8 +124,74 @@ void oracle_f32_to_bf16(uint16_t *dst, const float *src, int64_t n)
 {
 	int64_t i;
 
+#pragma omp parallel for if (n > 1000000)
 	for (i = 0; i < n; i++)
 		dst[i] = oracle_bf16_rne(src[i]);
+}
+
+/* ---- comparison helpers of the full-size tests (plain arithmetic, nothing of the reference) ---- */
+
+/* 1 when the two byte ranges are equal. */
+int oracle_same_bytes(const void *a, const void *b, int64_t nbytes)
+{
+	const int64_t chunk = (int64_t)1 << 24;
+	const int64_t n_chunks = (nbytes + chunk - 1) / chunk;
+	int same = 1;
+	int64_t c;
+
+#pragma omp parallel for reduction(&& : same) if (n_chunks > 4)
+	for (c = 0; c < n_chunks; c++) {
+		const int64_t at = c * chunk;
+		const int64_t len = nbytes - at < chunk ? nbytes - at : chunk;
+
+		same = same && memcmp((const char *)a + at, (const char *)b + at, (size_t)len) == 0;
+	}
+	return same;
+}
+
+static double cmp_value(const void *x, int type, int64_t i)
+{
+	return type == ORACLE_BF16 ? (double)oracle_bf16_widen(((const uint16_t *)x)[i])
+	    : (double)((const float *)x)[i];
+}
+
+/*
+** a against b (float arrays, or bf16 bit patterns that are widened): out[0] = max over i of
+** |a-b| / max(|b|, rms(b)); out[1] = how many elements have |a-b| > tol * |b|; out[2] = the largest
+** |b| among those (0 when there is none).
+*/
+void oracle_compare(const void *a, const void *b, int type, int64_t n, double tol, double *out)
+{
+	double ss = 0.0, worst = 0.0, biggest = 0.0, floor_;
+	int64_t count = 0;
+	int64_t i;
+
+#pragma omp parallel for reduction(+ : ss) if (n > 1000000)
+	for (i = 0; i < n; i++) {
+		const double y = cmp_value(b, type, i);
+
+		ss += y * y;
+	}
+	floor_ = (n > 0 ? sqrt(ss / (double)n) : 0.0) + 1e-300;
+#pragma omp parallel for reduction(max : worst, biggest) reduction(+ : count) if (n > 1000000)
+	for (i = 0; i < n; i++) {
+		const double x = cmp_value(a, type, i);
+		const double y = cmp_value(b, type, i);
+		const double d = fabs(x - y);
+		const double ay = fabs(y);
+		const double r = d / (ay > floor_ ? ay : floor_);
+
+		if (r > worst || r != r)
+			worst = r != r ? INFINITY : r;
+		if (d > tol * ay || d != d) {
+			count++;
+			if (ay > biggest)
+				biggest = ay;
+		}
+	}
+	out[0] = worst;
+	out[1] = (double)count;
+	out[2] = biggest;
 }
 
 /* ---- learning-rate schedule (lang/lm_train.c:98-124) ------------------ */

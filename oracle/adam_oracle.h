@@ -20,7 +20,7 @@
 **                                  (bias / LayerNorm gradients as serial float column sums)
 **
 ** Pinned by: the reference's compiled lm_adam_step_scaled (oracle/_ref, bit for
-** bit on p/m/v), the golden vectors it wrote (tests/golden/*.npz: oracle_adam_step_scaled
+** bit on p/m/v), the golden vectors it wrote (the .npz files under tests/golden: oracle_adam_step_scaled
 ** and oracle_adam_step_slots, bit for bit), the reference's own LR known answers
 ** (tests/test_ann.c:866-879), closed forms (t=1, constant gradient, zero gradient), and
 ** brute-force exact sums; oracle_colsum_add by the reference's compiled layernorm_backward
@@ -129,6 +129,14 @@ void	oracle_adam_step_slots(oracle_slot *slots, int64_t n, int t, double beta1,
 
 /* acc[j] += column sums of x (y != NULL: of x * y), rows x cols row-major, the host loops' order. */
 void	oracle_colsum_add(float *acc, const float *x, const float *y, int64_t rows, int cols);
+
+/*
+** Comparison helpers of the full-size tests: byte equality, and a against b with
+** out[0] = max |a-b| / max(|b|, rms(b)), out[1] = number of elements with |a-b| > tol * |b|,
+** out[2] = the largest |b| among those.  type ORACLE_F32 or ORACLE_BF16 (bit patterns, widened).
+*/
+int	oracle_same_bytes(const void *a, const void *b, int64_t nbytes);
+void	oracle_compare(const void *a, const void *b, int type, int64_t n, double tol, double *out);
 
 int	oracle_max_threads(void);
 

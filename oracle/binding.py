@@ -161,6 +161,31 @@ def bf16_rne(x):
     return out
 
 
+def same_bytes(a, b):
+    """True when two arrays of the same size hold the same bytes (threaded memcmp)."""
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    if a.nbytes != b.nbytes:
+        return False
+    L = lib()
+    L.oracle_same_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+    L.oracle_same_bytes.restype = C.c_int
+    return bool(L.oracle_same_bytes(_ptr(a), _ptr(b), a.nbytes))
+
+
+def compare(a, b, tol):
+    """a against b, float32 arrays or bf16 bit patterns (uint16): (max |a-b| / max(|b|, rms(b)),
+    number of elements with |a-b| > tol*|b|, the largest |b| among those)."""
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    assert a.dtype == b.dtype and a.size == b.size and a.dtype in (np.float32, np.uint16)
+    L = lib()
+    L.oracle_compare.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_double,
+                                 C.POINTER(C.c_double)]
+    L.oracle_compare.restype = None
+    out = (C.c_double * 3)()
+    L.oracle_compare(_ptr(a), _ptr(b), BF16 if a.dtype == np.uint16 else F32, a.size, tol, out)
+    return out[0], int(out[1]), out[2]
+
+
 def bf16_widen(h):
     return (h.astype(np.uint32) << 16).view(np.float32)
 

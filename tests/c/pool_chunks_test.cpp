@@ -78,6 +78,21 @@ int main(void)
 			held.erase(held.begin() + (long)k);
 			gives++;
 		}
+		/* now and then: reserve the largest free block whole (what the placement search uses as scratch) and hand it back */
+		if (op % 97 == 0) {
+			size_t big = 0;
+			const size_t at = c.largest_free(&big);
+
+			if (big > 0) {
+				if (c.take_block(at + 1) != 0) { printf("FAIL: take_block of an interior offset\n"); return 1; }
+				if (c.take_block(at) != big) { printf("FAIL: take_block\n"); return 1; }
+				if (c.take_block(at) != 0) { printf("FAIL: take_block of a used block\n"); return 1; }
+				memset(&map[at], 1, big);
+				check(c, map);
+				if (c.give(at) != big) { printf("FAIL: give after take_block\n"); return 1; }
+				memset(&map[at], 0, big);
+			}
+		}
 		check(c, map);
 	}
 	while (!held.empty()) { c.give(held.back().first); held.pop_back(); }

@@ -19,6 +19,9 @@ def same_bits(a, b):
     return a.shape == b.shape and bool((bits(a) == bits(b)).all())
 
 
+CHUNK = 1 << 26          # elements per pass of the full-size comparisons (keeps temporaries small)
+
+
 def rel_err(a, b):
     """max |a-b| / max(|b|, rms(b)), in double.
 
@@ -32,10 +35,35 @@ def rel_err(a, b):
     """
     if not a.size:
         return 0.0
-    a = a.astype(np.float64)
-    b = b.astype(np.float64)
-    floor = float(np.sqrt(np.mean(b * b))) + 1e-300
-    return float(np.max(np.abs(a - b) / np.maximum(np.abs(b), floor)))
+    a, b = a.reshape(-1), b.reshape(-1)
+    ss = 0.0
+    for at in range(0, b.size, CHUNK):
+        y = b[at:at + CHUNK].astype(np.float64)
+        ss += float(np.dot(y, y))
+    floor = float(np.sqrt(ss / b.size)) + 1e-300
+    worst = 0.0
+    for at in range(0, b.size, CHUNK):
+        x = a[at:at + CHUNK].astype(np.float64)
+        y = b[at:at + CHUNK].astype(np.float64)
+        worst = max(worst, float(np.max(np.abs(x - y) / np.maximum(np.abs(y), floor))))
+    return worst
+
+
+def strict_misses(a, b, tol):
+    """The letter of "within tol relative": how many elements have |a-b| > tol*|b|, and the
+    largest |b| among them (0.0 when there is none).  See rel_err for why some must exist when the
+    two sides used clip norms that differ in their last bits: they are the cancelling ones."""
+    a, b = a.reshape(-1), b.reshape(-1)
+    count, biggest = 0, 0.0
+    for at in range(0, b.size, CHUNK):
+        x = a[at:at + CHUNK].astype(np.float64)
+        y = np.abs(b[at:at + CHUNK].astype(np.float64))
+        bad = np.abs(x - b[at:at + CHUNK].astype(np.float64)) > tol * y
+        k = int(np.count_nonzero(bad))
+        if k:
+            count += k
+            biggest = max(biggest, float(y[bad].max()))
+    return count, biggest
 
 
 def bf16_ulp_diff(a_u16, b_u16):

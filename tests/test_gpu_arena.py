@@ -596,3 +596,137 @@ def test_bf16_conversion_on_all_float_patterns(gpu, oracle):
         assert bad.size == 0, [(hex(int(bits[i])), hex(int(got[i]))) for i in bad[:4]]
     src.free()
     dst.free()
+
+
+@pytest.mark.parametrize("mode", ["f32", "bf16"])
+def test_moments_offloaded_between_steps(gpu, oracle, mode):
+    """anni_adam_set_offload (lm_adam_set_offload, lang/lm_adam.c:211-214,295-334): after every step
+    m and v leave the device for page-locked host memory and their blocks are given back, the next
+    step brings them back first.  Same bits as the oracle at every step; the moments really are
+    gone in between (NULL pointers, and device memory in use reads the same after every step);
+    the checkpoint calls still see them; switching it off brings them back for good."""
+    import ctypes as C
+    narrow = 1 if mode == "bf16" else 0
+    tensors = [(80 * 1000 * 1000, 3), (4097, 0), (12288, 3), (3, 1)]      # flats of 160 - 320 MB: pooled blocks
+    opt = make(gpu, tensors, grad_type=0, moment_type=narrow, beta2=0.95, weight_decay=0.1,
+               grad_clip=1.0, skip_nonfinite=True)
+    n = opt.n
+    rng = np.random.default_rng(11)
+    P = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    opt.upload("param", P)
+    opt.seed_twins()
+    mt = oracle.BF16 if narrow else oracle.F32
+    M, V = (np.zeros(n, np.uint16), np.zeros(n, np.uint16)) if narrow else \
+        (np.zeros(n, np.float32), np.zeros(n, np.float32))
+    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True,
+                      moment_type=mt, tensors=oracle_tensors(opt), threads=8)
+    unit = 1.0 / (np.sqrt(n) * 1e-3)
+
+    def one_step(s):
+        g = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+        opt.upload("grad", g)
+        gs = unit * (1.7 if s % 2 else 0.6)
+        assert opt.step_scaled(1e-3, gs) == 0
+        st = opt.sync_stats()
+        O.step(P, g, M, V, 1e-3, gs, sumsq_override=st.last_sumsq)
+        assert st.last_clipped == s % 2
+        assert same_bits(opt.download("param"), P), s
+        assert (opt.download("twin")[twin_mask(opt)] == oracle.bf16_rne(P)[twin_mask(opt)]).all()
+
+    one_step(0)                                              # a step before the switch: m, v non-zero
+    old = (opt.o.d_param, opt.o.d_m)
+    assert gpu.anni_adam_mv_on_device(opt.h) == 1
+    assert gpu.anni_adam_set_offload(opt.h, 1) == 0, gpu.gpu_debug_last_error()
+    assert gpu.anni_adam_mv_on_device(opt.h) == 0 and not opt.o.d_m and not opt.o.d_v
+    assert opt.o.d_param and opt.o.d_param != old[0]         # the arena was re-housed without m and v
+    fr0, tt = C.c_size_t(0), C.c_size_t(0)
+    assert gpu.gpu_mem_info(C.byref(fr0), C.byref(tt)) == 0
+    for s in range(1, 4):
+        one_step(s)
+        assert gpu.anni_adam_mv_on_device(opt.h) == 0
+        fr = C.c_size_t(0)
+        assert gpu.gpu_mem_info(C.byref(fr), C.byref(tt)) == 0
+        assert fr.value == fr0.value, "device memory in use moved between steps"
+    pairs = opt.export_mv(0, 5000)                           # brings them back, sends them away again
+    wide = (lambda a: oracle.bf16_widen(a)) if narrow else (lambda a: a)
+    assert same_bits(pairs[:, 0].copy(), wide(M[:5000])) and same_bits(pairs[:, 1].copy(), wide(V[:5000]))
+    assert gpu.anni_adam_mv_on_device(opt.h) == 0
+    assert gpu.anni_adam_set_offload(opt.h, 0) == 0
+    assert gpu.anni_adam_mv_on_device(opt.h) == 1 and opt.o.d_m and opt.o.d_v
+    got_m, got_v = opt.download("m"), opt.download("v")
+    assert (got_m.view(M.dtype) == M).all() if narrow else same_bits(got_m, M)
+    assert (got_v.view(V.dtype) == V).all() if narrow else same_bits(got_v, V)
+    one_step(4)                                              # and on it goes, moments resident again
+    assert gpu.anni_adam_mv_on_device(opt.h) == 1
+    opt.free()
+
+
+def test_sum_of_squares_self_check_runs_once_and_agrees(gpu, oracle):
+    """The first sum of squares with a second stage compares its atomic hand-over of the partials
+    with the fenced one on the caller's own gradients (two extra launches, one wait); so does the
+    first one after the switches were read again.  The two never disagree here, and the fenced
+    form selected by hand gives the same bits as the default."""
+    import ctypes as C
+    import os
+    runs0, bad0 = C.c_int(0), C.c_int(0)
+    opt = make(gpu, [(4096 * 2300 + 77, 3), (513, 0)], beta2=0.95, grad_clip=1.0, skip_nonfinite=True)
+    n = opt.n
+    rng = np.random.default_rng(12)
+    g = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    opt.upload("grad", g)
+    assert opt.step_scaled(1e-3) == 0
+    st = opt.sync_stats()
+    want = st.last_sumsq
+    assert gpu.anni_fold_guard_stats(C.byref(runs0), C.byref(bad0)) == 0
+    assert runs0.value >= 1 and bad0.value == 0
+    opt.upload("grad", g)
+    assert opt.step_scaled(1e-3) == 0                       # no second check
+    runs1, bad1 = C.c_int(0), C.c_int(0)
+    gpu.anni_fold_guard_stats(C.byref(runs1), C.byref(bad1))
+    assert runs1.value == runs0.value and opt.sync_stats().last_sumsq == want
+    try:
+        os.environ["ANNI_FOLD"] = "fence"
+        gpu.anni_gpu_reload_switches()
+        opt.upload("grad", g)
+        assert opt.step_scaled(1e-3) == 0
+        assert opt.sync_stats().last_sumsq == want          # the fenced form, same bits
+        gpu.anni_fold_guard_stats(C.byref(runs1), C.byref(bad1))
+        assert runs1.value == runs0.value                   # nothing to check it against
+    finally:
+        os.environ.pop("ANNI_FOLD", None)
+        gpu.anni_gpu_reload_switches()
+    opt.upload("grad", g)
+    assert opt.step_scaled(1e-3) == 0                       # read again: checked again
+    gpu.anni_fold_guard_stats(C.byref(runs1), C.byref(bad1))
+    assert runs1.value == runs0.value + 1 and bad1.value == 0
+    assert opt.sync_stats().last_sumsq == want
+    assert abs(want - oracle.sumsq(g, threads=4)) <= 1e-10 * want
+    opt.free()
+
+
+def test_gnorm_every_alone_computes_and_prints_the_norm(gpu):
+    """lm_adam.c:466,484-487: with ANN_GNORM_EVERY=N the norm is computed and printed every N steps
+    also when nothing clips and nothing skips (the switch is read once per process: a child)."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    child = (
+        "import sys; sys.path.insert(0, %r)\n"
+        "import numpy as np\n"
+        "from anni_amd.lm_adam import LmAdam\n"
+        "opt = LmAdam([(5000, 3), (77, 0)])\n"
+        "for s in range(4):\n"
+        "    opt.upload('grad', np.full(opt.n, 0.5, np.float32))\n"
+        "    opt.step_scaled(1e-3)\n"
+        "    st = opt.sync_stats()\n"
+        "    print('NORM %%d %%r %%d' %% (opt.t, st.last_grad_norm, st.last_clipped))\n"
+    ) % root
+    env = dict(os.environ, ANN_GNORM_EVERY="2")
+    r = subprocess.run([sys.executable, "-c", child], env=env, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr[-1500:]
+    want = float(np.sqrt(5077 * 0.25))
+    norms = [ln.split() for ln in r.stdout.splitlines() if ln.startswith("NORM ")]
+    assert len(norms) == 4 and all(abs(float(x[2]) - want) < 1e-9 * want and x[3] == "0" for x in norms)
+    said = [ln for ln in r.stderr.splitlines() if ln.startswith("[adam] step ")]
+    assert said == ["[adam] step 2 grad norm %.4g" % want, "[adam] step 4 grad norm %.4g" % want], r.stderr

@@ -598,3 +598,52 @@ def test_malloc_and_free_from_many_threads(gpu):
     assert gpu.gpu_mem_info(C.byref(fr1), C.byref(tt)) == 0
     assert abs(fr1.value - fr0.value) <= 64 << 20    # the runtime's own pools may have grown a little
     gpu.gpu_free(hold)
+
+
+def test_grad_sumsq_from_two_threads_is_right_or_refused(gpu, oracle):
+    """gpu_grad_sumsq has one result slot per process (as the reference's static accumulator,
+    num/gpu_cuda.cu:8485-8486) and is meant for one thread.  A second call that arrives while one
+    is between its launch and its read-back is turned away with -1 -- it never returns the other
+    call's sum."""
+    import threading
+    from anni_amd.lm_adam import DeviceBuffer
+    rng = np.random.default_rng(77)
+    n = 6 * 1000 * 1000
+    xs = [(rng.standard_normal(n) * (k + 1)).astype(np.float32) for k in range(2)]
+    want = [oracle.sumsq(x, threads=4) for x in xs]
+    bufs = [DeviceBuffer(4 * n) for _ in xs]
+    for b, x in zip(bufs, xs):
+        b.upload(x)
+    results = [[], []]
+
+    def work(k):
+        out = C.c_double(0)
+        good = 0
+        for _ in range(200000):                            # until 60 calls got in (the other thread is in the way)
+            rc = gpu.gpu_grad_sumsq(bufs[k].ptr, n, C.byref(out))
+            results[k].append((rc, out.value))
+            good += rc == 0
+            if good == 60:
+                break
+    th = [threading.Thread(target=work, args=(k,)) for k in range(2)]
+    for t in th:
+        t.start()
+    for t in th:
+        t.join()
+    refused = 0
+    for k in range(2):
+        done = 0
+        for rc, val in results[k]:
+            assert rc in (0, -1)
+            if rc == 0:
+                assert abs(val - want[k]) <= 1e-10 * want[k], (k, val, want[k])
+                done += 1
+            else:
+                refused += 1
+        assert done == 60, (k, done, len(results[k]))
+    print("calls refused while the other thread was inside: %d" % refused, flush=True)
+    out = C.c_double(0)
+    assert gpu.gpu_grad_sumsq(bufs[0].ptr, n, C.byref(out)) == 0      # and the flag is free afterwards
+    assert abs(out.value - want[0]) <= 1e-10 * want[0]
+    for b in bufs:
+        b.free()

