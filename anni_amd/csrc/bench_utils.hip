@@ -13,7 +13,7 @@
 #include "anni_gpu.h"
 #include "anni_hooks.h"
 
-namespace {
+namespace anni_bench {
 
 constexpr int kLanes = 256;
 
@@ -59,7 +59,7 @@ __global__ __launch_bounds__(kLanes) void copy16_kernel(void *dst, const void *s
 		((u32x4 *)dst)[i] = ((const u32x4 *)src)[i];
 }
 
-int util_grid(int64_t items)
+static int util_grid(int64_t items)
 {
 	int64_t g = (items + kLanes - 1) / kLanes;
 
@@ -70,9 +70,9 @@ int util_grid(int64_t items)
 	return (int)g;
 }
 
-float g_last_derived_ms;	/* E4M3 pass time of the last per-kernel run of anni_adam_time_steps */
+static float g_last_derived_ms;	/* E4M3 pass time of the last per-kernel run of anni_adam_time_steps */
 
-int time_steps_body(anni_adam *opt, int count, void *const *grads, int n_grads, const double *lr,
+static int time_steps_body(anni_adam *opt, int count, void *const *grads, int n_grads, const double *lr,
 	const double *grad_scale, float *ms_total, float *ms_sumsq, float *ms_update)
 {
 	std::vector<hipEvent_t> ev;
@@ -160,7 +160,9 @@ int time_steps_body(anni_adam *opt, int count, void *const *grads, int n_grads, 
 	return rc;
 }
 
-} /* namespace */
+} /* namespace anni_bench */
+
+using namespace anni_bench;
 
 extern "C" {
 

@@ -170,7 +170,7 @@ def load():
                 "(or __graft_entry__.build()); there is no CPU fallback" % SO_PATH)
         if not os.path.exists(BENCH_SO_PATH):
             raise LibraryMissing("%s is missing: build it with `make -C anni_amd/csrc`" % BENCH_SO_PATH)
-        L = C.CDLL(SO_PATH, mode=C.RTLD_GLOBAL)
+        L = C.CDLL(SO_PATH)
         B = C.CDLL(BENCH_SO_PATH)
         for lib_, protos in ((L, _PROTOS), (B, _BENCH_PROTOS)):
             for name, (res, args) in protos.items():

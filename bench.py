@@ -337,22 +337,26 @@ def cpu_baselines(size_name, norm_bpp, upd_bpp, budget_s):
     return mt_out, serial_out
 
 
-def reference_caller_leg(L, size="185m"):
+def reference_caller_leg(L, size="185m", call_trace=False):
     """The reference's own lm + lm_adam_create + lm_adam_step_scaled (compiled from the reference
     tree, linked against this backend) timed wall-clock per step: at its compile-time size
     (oracle/_ref/libanni_ref_hip.so: untied 16384-token embedding) or, size "555m", at the sizes of
     its 555M run with the tied 100000-token embedding (oracle/_ref/libanni_ref_555m_hip.so).
+    call_trace: the flavours with the call-timing interposer in front of the backend
+    (oracle/gputrace.c); the last step's calls are reported as a host-side timeline.
     None when that library did not travel."""
     from oracle import binding as ob
+    have = ob.ref_trace_available() if call_trace else \
+        (ob.ref_hip_available() if size == "185m" else ob.ref_hip_555m_available())
+    if not have:
+        return None
+    suffix = "_trace" if call_trace else ""
     if size == "185m":
-        if not ob.ref_hip_available():
-            return None
-        make = lambda: ob.RefModelOnBackend(16384, beta2=0.95, weight_decay=0.1, grad_clip=1.0)
+        make = lambda: ob.RefModelOnBackend(16384, beta2=0.95, weight_decay=0.1, grad_clip=1.0,
+                                            backend="hip" + suffix)
     else:
-        if not ob.ref_hip_555m_available():
-            return None
         make = lambda: ob.RefModelOnBackend(100000, beta2=0.95, weight_decay=0.1, grad_clip=1.0,
-                                            backend="hip555m", tied=True)
+                                            backend="hip555m" + suffix, tied=True)
     L.gpu_set_compute_prec(1)
     M = make()
     n = M.n
@@ -361,25 +365,67 @@ def reference_caller_leg(L, size="185m"):
     g = rng.standard_normal(n, dtype=np.float32) * np.float32(1e-3)
     unit = 1.0 / (math.sqrt(n) * 1e-3)
     times = []
-    for t in range(1, 10):
+    last = 9
+    for t in range(1, last + 1):
         M.set_grads(g)
         L.gpu_device_sync()
+        if call_trace and t == last:
+            ob.gputrace().gputrace_start()
         t0 = time.perf_counter()
         M.step(3e-6 * t, unit * (1.7 if t % 2 else 0.6))
         times.append((time.perf_counter() - t0) * 1e3)
+        if call_trace:
+            ob.gputrace().gputrace_stop()
     n_segs = M.n_segs
+    events = ob.gputrace_events() if call_trace else None
     M.close()
     L.gpu_set_compute_prec(0)
     L.gpu_adam_set_weight_decay(0.0)
     ms = float(np.median(times[1:]))
-    return {"what": "unchanged lang/lm_adam.c (lm_adam_step_scaled, device path) on this backend: "
-                    "matrices aliased into the flats, bias/LayerNorm vectors host-resident (uploaded "
-                    "before and read back after every step by the caller), norm read back by the caller",
-            "params": n, "segments": n_segs, "host_vector_bytes": vec_bytes,
-            "ms_per_step": round(ms, 3), "min_ms": round(min(times[1:]), 3),
-            "first_step_ms_with_arena_init": round(times[0], 1),
-            "GBps_algorithmic": round(n * 38 / ms / 1e6, 1),
-            "frac": round(n * 38 / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    out = {"what": "unchanged lang/lm_adam.c (lm_adam_step_scaled, device path) on this backend: "
+                   "matrices aliased into the flats, bias/LayerNorm vectors host-resident (uploaded "
+                   "before and read back after every step by the caller), norm read back by the caller",
+           "params": n, "segments": n_segs, "host_vector_bytes": vec_bytes,
+           "ms_per_step": round(ms, 3), "min_ms": round(min(times[1:]), 3),
+           "first_step_ms_with_arena_init": round(times[0], 1),
+           "GBps_algorithmic": round(n * 38 / ms / 1e6, 1),
+           "frac": round(n * 38 / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    if events:
+        out["call_trace_of_the_last_step"] = call_timeline(events, times[-1])
+    return out
+
+
+def call_timeline(ev, wall_ms):
+    """Host-side timeline of one lm_adam_step_scaled from the interposer's records (microseconds)."""
+    base = ev[0][1]
+    per = {}
+    for nm, a, b, by in ev:
+        k = per.setdefault(nm, [0, 0.0, 0])
+        k[0] += 1
+        k[1] += b - a
+        k[2] += by
+
+    def first(nm):
+        return next(i for i, e in enumerate(ev) if e[0] == nm)
+    i_ss, i_st = first("gpu_grad_sumsq"), first("gpu_adam_step_dev_bf16")
+    i_sy = max(i for i, e in enumerate(ev) if e[0] == "gpu_stream_sync")
+    r = lambda x: round(x, 1)
+    return {
+        "wall_ms_with_interposer": round(wall_ms, 3), "calls": len(ev),
+        "per_entry_point_us": {nm: {"calls": c, "total_us": r(us), "bytes": by}
+                               for nm, (c, us, by) in sorted(per.items(), key=lambda kv: -kv[1][1]) if us >= 0.05},
+        "callers_own_time_between_calls_us": r(sum(ev[i + 1][1] - ev[i][2] for i in range(len(ev) - 1))),
+        "phases_us": {
+            "gather: step start .. gpu_grad_sumsq called (the caller stages its vectors; device idle "
+            "but for the copy pieces)": r(ev[i_ss][1] - base),
+            "gpu_grad_sumsq (last copy piece, sum of squares, wait, read-back)": r(ev[i_ss][2] - ev[i_ss][1]),
+            "norm on the host .. update launched": r(ev[i_st][2] - ev[i_ss][2]),
+            "scatter calls (queued behind the update)": r(ev[i_sy][1] - ev[i_st][2]),
+            "gpu_stream_sync (rest of the update, copy-back kernel, wait, hand-over to the caller's vectors)":
+                r(ev[i_sy][2] - ev[i_sy][1]),
+            "after": r(ev[-1][2] - ev[i_sy][2])},
+        "calls_over_10us": [{"entry": nm, "at_us": r(a - base), "us": r(b - a), "bytes": by}
+                            for nm, a, b, by in ev if b - a > 10.0]}
 
 
 def colsum_leg(L, rows, shapes=((6272, False), (1536, False), (1536, True))):
@@ -645,6 +691,10 @@ def main():
                     help="only measure what the search for the arena's second block costs and leaves behind")
     ap.add_argument("--reference-caller-only", action="store_true",
                     help="only time the unchanged reference caller on this backend (one JSON line)")
+    ap.add_argument("--ref-size", default="both", choices=["185m", "555m", "both"],
+                    help="with --reference-caller-only: which of the two compiled sizes of the reference to run")
+    ap.add_argument("--call-trace", action="store_true",
+                    help="with --reference-caller-only: time every backend call of one step through the interposer")
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds for the CPU legs")
     ap.add_argument("--derived", nargs="?", const="both", default=None,
                     choices=["both", "fp8", "pack"],
@@ -688,8 +738,8 @@ def main():
         print(json.dumps({"placement_cost": placement_cost_leg(L)}))
         return
     if a.reference_caller_only:
-        print(json.dumps({"reference_caller_185m": reference_caller_leg(L, "185m"),
-                          "reference_caller_555m": reference_caller_leg(L, "555m")}))
+        print(json.dumps({"reference_caller_" + sz: reference_caller_leg(L, sz, a.call_trace)
+                          for sz in ("185m", "555m") if a.ref_size in (sz, "both")}))
         return
 
     size, gt, mt, norm_bpp, upd_bpp = WORKLOADS[a.workload]
@@ -871,17 +921,8 @@ def main():
         out["gpu_over_cpu"] = round(step_gbps / mt_out["value"], 1)
     opt.free()
     opt = None
-    if a.workload == "555m" and not a.derived and not a.no_legs:
-        # the same workload with every flat in ONE allocation, and the other parameter set the
-        # metric names, each on an arena of its own after the headline's was freed
-        try:
-            out["layout_compact"] = short_leg(L, "555m", "compact")
-            out["workloads"] = {}
-            for w in ("185m", "555m-bf16", "1p4b-fp8"):
-                out["workloads"][w] = short_leg(L, w, "auto")
-        except Exception as e:                      # a side leg must never sink the bench line
-            out["side_legs_error"] = repr(e)
-    if not a.no_cpu:
+    if not a.no_cpu and not a.no_legs:
+        # the unchanged reference caller on this backend, right after the headline's arena was freed
         try:
             for size in ("185m", "555m"):
                 ref_leg = reference_caller_leg(L, size)
@@ -889,6 +930,16 @@ def main():
                     out["reference_caller_" + size] = ref_leg
         except Exception as e:                      # the checker must never sink the bench line
             out["reference_caller_error"] = repr(e)
+    if a.workload == "555m" and not a.derived and not a.no_legs:
+        # the same workload with every flat in ONE allocation, and the other configurations the
+        # metric names, each on an arena of its own after the one before it was freed
+        try:
+            out["layout_compact"] = short_leg(L, "555m", "compact")
+            out["workloads"] = {}
+            for w in ("185m", "555m-bf16", "1p4b-fp8"):
+                out["workloads"][w] = short_leg(L, w, "auto")
+        except Exception as e:                      # a side leg must never sink the bench line
+            out["side_legs_error"] = repr(e)
     if a.ref_jsonl:
         row = bench_row.adam_row(env, a.workload, size, gt, mt, n, a.warmup, per_step_ms, 3e-4,
                                  peak_mb, not skipped_steps)

@@ -368,6 +368,53 @@ def ref_hip_555m():
     return _ref_hip_555m
 
 
+# The same two flavours with the call-timing interposer (gputrace.c) linked in front of the backend.
+REF_TRACE_SO = {"hip_trace": os.path.join(HERE, "_ref", "libanni_ref_hip_trace.so"),
+                "hip555m_trace": os.path.join(HERE, "_ref", "libanni_ref_555m_hip_trace.so")}
+GPUTRACE_SO = os.path.join(HERE, "_ref", "libgputrace.so")
+_ref_trace = {}
+_gputrace = None
+
+
+def ref_trace_available():
+    return os.path.exists(GPUTRACE_SO) and all(os.path.exists(p) for p in REF_TRACE_SO.values())
+
+
+def ref_trace(flavour):
+    """The traced flavour "hip_trace" / "hip555m_trace" of the compiled reference."""
+    if flavour not in _ref_trace:
+        os.environ.setdefault("ANNI_HIP_SO", os.path.join(os.path.dirname(HERE), "anni_amd",
+                                                          "libanni_gpu_hip.so"))
+        R = C.CDLL(REF_TRACE_SO[flavour])
+        _declare_model(R)
+        _ref_trace[flavour] = R
+    return _ref_trace[flavour]
+
+
+def gputrace():
+    """The interposer's own entry points: start / stop recording, and the recorded calls."""
+    global _gputrace
+    if _gputrace is None:
+        T = C.CDLL(GPUTRACE_SO)
+        T.gputrace_get.argtypes = [C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_double),
+                                   C.POINTER(C.c_double), C.POINTER(C.c_size_t)]
+        T.gputrace_name.restype = C.c_char_p
+        T.gputrace_name.argtypes = [C.c_int]
+        _gputrace = T
+    return _gputrace
+
+
+def gputrace_events():
+    """[(name, start us, end us, bytes)] of the calls recorded since gputrace_start."""
+    T = gputrace()
+    out = []
+    for i in range(T.gputrace_count()):
+        a, b, c, d = C.c_int(), C.c_double(), C.c_double(), C.c_size_t()
+        T.gputrace_get(i, C.byref(a), C.byref(b), C.byref(c), C.byref(d))
+        out.append((T.gputrace_name(a.value).decode(), b.value, c.value, d.value))
+    return out
+
+
 _ref_cpu_model = None
 
 
@@ -392,7 +439,7 @@ class RefModelOnBackend:
     def __init__(self, vocab=16384, beta2=0.95, weight_decay=0.1, grad_clip=1.0, backend="hip",
                  _handle=None, tied=False):
         self.R = (ref_hip() if backend == "hip" else ref_hip_555m() if backend == "hip555m"
-                  else ref_cpu_model_lib())
+                  else ref_trace(backend) if backend in REF_TRACE_SO else ref_cpu_model_lib())
         create = self.R.ref_model_create_tied if tied else self.R.ref_model_create
         self.h = _handle or create(vocab, beta2, weight_decay, grad_clip)
         if not self.h:
