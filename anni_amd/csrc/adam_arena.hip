@@ -1494,9 +1494,30 @@ void anni_hook_reload_switches(void)
 	reload_switches();
 }
 
-void anni_hook_fold_guard_stats(int *runs, int *mismatches)
+long anni_hook_counter(const char *name)
 {
-	fold_guard_stats(runs, mismatches);
+	int runs = 0, bad = 0;
+	long used = 0, dropped = 0;
+
+	if (!name)
+		return -1;
+	fold_guard_stats(&runs, &bad);
+	early_sum_stats(&used, &dropped);
+	if (strcmp(name, "fold_guard_runs") == 0)
+		return runs;
+	if (strcmp(name, "fold_guard_mismatches") == 0)
+		return bad;
+	if (strcmp(name, "early_sum_used") == 0)
+		return used;
+	if (strcmp(name, "early_sum_dropped") == 0)
+		return dropped;
+	if (strcmp(name, "vectors_first_steps") == 0 || strcmp(name, "vectors_first_served") == 0) {
+		long steps = 0, served = 0;
+
+		vectors_first_stats(&steps, &served);
+		return strcmp(name, "vectors_first_steps") == 0 ? steps : served;
+	}
+	return -1;
 }
 
 int anni_gpu_device_info(char *name, size_t cap, int *driver_version)

@@ -140,6 +140,41 @@ int	launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *parti
 int	launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double grad_scale,
 		const NormIn &norm);
 /*
+** The same update for the tiles (kTile elements each) order[0 .. turns) only, in that order;
+** `order` is device memory.  Two such launches over disjoint tiles may run side by side.  -1 when
+** the storage mode would take a software-pipelined kernel, which has no such form.
+*/
+int	update_walks_backwards(void);	/* launch_update takes the tiles from the last to the first */
+int	launch_update_tiles(hipStream_t st, const Flat &f, const StepConsts &c, double grad_scale,
+		const NormIn &norm, const int32_t *order, int64_t turns);
+/*
+** The sum of squares of a float flat in separable steps (the flat entry point gpu_grad_sumsq):
+** launch_chunk_sums writes kWaves partial sums for every 16 KiB chunk of x (list == NULL) or for
+** the n_list chunks named in `list` (device-readable memory) into part[chunk * kWaves ..];
+** launch_chunk_fold adds all chunk_sums_count(n) * kWaves partials in index order, through at
+** most kChunkRuns intermediate sums in `runs`, and stores {sum, sqrt(sum), 1, 0, 0} into *state.
+** The sum is a function of x alone: partials recomputed for some chunks after their elements
+** changed give the bits a pass over the whole flat would.
+*/
+constexpr int kChunkRuns = 1024;
+int	chunk_sums_count(int64_t n);
+int	launch_chunk_sums(hipStream_t st, const float *x, int64_t n, double *part, const int32_t *list,
+		int n_list);
+int	launch_chunk_fold(hipStream_t st, const double *part, int64_t n, double *runs, StepState *state);
+/*
+** The end of the sum in one launch: the partials of the n_fix chunks in `fix` (rising, no chunk
+** twice; host memory, `fix_dev` the same list where the device can read it) are computed anew,
+** then everything is folded as launch_chunk_fold does, with the same bits.  ticket: kTicketBytes
+** of zeroed device memory, 128-byte aligned, left zeroed.  The first call per device checks the
+** one launch against the separate kernels and waits for the stream once; calls must not overlap.
+** stamp (may be NULL; page-locked host memory): receives `token` after *state has been stored, for
+** a host that would rather watch a word than wait for the stream.  Returns 0 when the stamp will
+** be written, 1 when the launch went the way of the separate kernels, which write none, -1 on error.
+*/
+int	launch_chunk_finish(hipStream_t st, const float *x, int64_t n, double *part, const int32_t *fix,
+		const int32_t *fix_dev, int n_fix, double *runs, unsigned int *ticket, StepState *state,
+		unsigned long long *stamp, unsigned long long token);
+/*
 ** Derived outputs straight from p, without an update (after weights were loaded):
 ** wamax and the packed matrices as the update would leave them.
 */

@@ -528,6 +528,228 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(SumsqArgs a)
 	sumsq_finish(a, total, lds, &last);
 }
 
+/* ---- sum of squares of a float flat, one partial per wavefront and chunk --------------- */
+
+/*
+** The flat entry point (gpu_grad_sumsq) sums in two steps that can be taken apart: first every
+** 16 KiB chunk of the flat gets four partial sums, one per wavefront of the workgroup that read
+** it (shuffles only, no barrier), then the partials are folded in index order -- chunk_fold_kernel
+** over contiguous runs, chunk_final_kernel over the runs' sums.  The result is a pure function of
+** the flat: it does not depend on the grid, and recomputing the partials of some chunks after
+** their elements changed gives bit for bit what a pass over the whole flat gives.  That is what
+** lets the backend begin the sum before the caller asks for it (gpu_backend.hip, "the sum begun
+** early") and repair the few chunks the caller still writes afterwards.
+*/
+struct ChunkSumArgs {
+	const float	*x;
+	int64_t		n;
+	double		*part;		/* kWaves per chunk */
+	const int32_t	*list;		/* NULL: every chunk; else the chunks to (re)compute, one per workgroup */
+	int		n_list;
+	int		vec_ok;
+	int64_t		keep_from;	/* chunks from here on are read with ordinary (cacheable) loads */
+};
+
+template <bool NT>
+__device__ __forceinline__ double chunk_sum_lane(const ChunkSumArgs &a, int64_t c, int tid)
+{
+	typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+	constexpr int64_t kElems = SumsqChunk<kF32>::kElems;
+	const int64_t base = c * kElems;
+	double acc[4] = {0.0, 0.0, 0.0, 0.0};
+
+	if (a.vec_ok && base + kElems <= a.n) {
+		const u32x4 *src = (const u32x4 *)(a.x + base) + tid;
+		u32x4 W[4];
+
+#pragma unroll
+		for (int u = 0; u < 4; u++)
+			W[u] = ld<NT>(src + u * kThreads);
+#pragma unroll
+		for (int u = 0; u < 4; u++) {
+#pragma unroll
+			for (int k = 0; k < 4; k++) {
+				const double v = (double)__uint_as_float(W[u][k]);
+
+				acc[k] += v * v;
+			}
+		}
+	} else {
+		const int64_t end = base + kElems < a.n ? base + kElems : a.n;
+
+		for (int64_t i = base + tid; i < end; i += kThreads) {
+			const double v = (double)a.x[i];
+
+			acc[0] += v * v;
+		}
+	}
+	return (acc[0] + acc[1]) + (acc[2] + acc[3]);
+}
+
+template <bool NT>
+__global__ __launch_bounds__(kThreads) void chunk_sums_kernel(ChunkSumArgs a)
+{
+	constexpr int64_t kElems = SumsqChunk<kF32>::kElems;
+	const int tid = threadIdx.x;
+	const int64_t n_chunks = (a.n + kElems - 1) / kElems;
+	const int64_t first = a.list ? 0 : blockIdx.x;
+	const int64_t step = a.list ? 1 : gridDim.x;
+	const int64_t stop = a.list ? 1 : n_chunks;
+
+	/*
+	** (Keeping the loads of a workgroup's next chunk in flight while it folds the current one was
+	** measured no faster: 0.389 against 0.381 ms per call at 555M.)
+	*/
+	for (int64_t k = first; k < stop; k += step) {
+		const int64_t c = a.list ? (int64_t)a.list[blockIdx.x] : k;
+		double x;
+
+		if (c < 0 || c >= n_chunks)
+			continue;
+		x = (NT && c < a.keep_from) ? chunk_sum_lane<true>(a, c, tid) : chunk_sum_lane<false>(a, c, tid);
+#pragma unroll
+		for (int off = 32; off > 0; off >>= 1)
+			x += __shfl_down(x, off, 64);
+		if ((tid & 63) == 0)
+			a.part[c * kWaves + (tid >> 6)] = x;
+	}
+}
+
+/* run[g] = sum of part[g * per .. min((g + 1) * per, count)) : lane l adds every 256th, then the fixed tree. */
+__global__ __launch_bounds__(kThreads) void chunk_fold_kernel(const double *part, int64_t count, int64_t per,
+	double *run)
+{
+	__shared__ double lds[4];
+	const int64_t lo = (int64_t)blockIdx.x * per;
+	const int64_t hi = lo + per < count ? lo + per : count;
+	double acc = 0.0;
+
+	for (int64_t i0 = lo + threadIdx.x; i0 < hi; i0 += (int64_t)kFoldAhead * kThreads) {
+		double v[kFoldAhead];
+
+#pragma unroll
+		for (int k = 0; k < kFoldAhead; k++) {
+			const int64_t i = i0 + (int64_t)k * kThreads;
+
+			v[k] = i < hi ? part[i] : 0.0;
+		}
+#pragma unroll
+		for (int k = 0; k < kFoldAhead; k++)
+			if (i0 + (int64_t)k * kThreads < hi)
+				acc += v[k];
+	}
+	const double total = block_sum(acc, lds);
+
+	if (threadIdx.x == 0)
+		run[blockIdx.x] = total;
+}
+
+/* The runs' sums in index order -> the state (state may lie in page-locked host memory). */
+__global__ __launch_bounds__(kThreads) void chunk_final_kernel(const double *run, int n_runs, StepState *state)
+{
+	__shared__ double lds[4];
+	double acc = 0.0;
+
+	for (int i = threadIdx.x; i < n_runs; i += kThreads)
+		acc += run[i];
+	const double ss = block_sum(acc, lds);
+
+	(void)norm_decide(ss, 0.0, 0, 1.0, state, threadIdx.x == 0);
+}
+
+/*
+** The three kernels above in one launch, for a caller who waits for the result: every kernel
+** boundary on one stream costs about 10 us here.  Workgroup r owns run r.  It first computes anew
+** the partials of those chunks of its run that are named in `fix` (rising, at most kFixMax, in the
+** kernel's arguments), then folds its run exactly as chunk_fold_kernel does, then hands the run's
+** sum over as the sum of squares' second stage does (sumsq_finish): whoever draws the last ticket
+** folds the runs' sums as chunk_final_kernel does.  Same additions in the same order: same bits.
+** The partials a workgroup has just written are read back by its other wavefronts; both sides use
+** device-scope atomic accesses with the barrier between them, so no cache of a compute unit can
+** stand in between.
+*/
+constexpr int kFixMax = 768;
+
+struct ChunkFinishArgs {
+	ChunkSumArgs	sum;		/* list unused */
+	int64_t		count;		/* partials in all */
+	int64_t		per;		/* partials per run, a multiple of kWaves */
+	SumsqArgs	fin;		/* partials = the runs' sums, ticket, state, fence */
+	unsigned long long	*stamp;	/* may be NULL: receives `token` once the state is stored */
+	unsigned long long	token;
+	int		n_fix;
+	int32_t		fix[kFixMax];
+};
+
+template <bool NT>
+__global__ __launch_bounds__(kThreads) void chunk_finish_kernel(ChunkFinishArgs a)
+{
+	__shared__ double lds[4];
+	__shared__ int last;
+	unsigned long long *cells = (unsigned long long *)a.sum.part;
+	const int tid = threadIdx.x;
+	const int64_t lo = (int64_t)blockIdx.x * a.per;
+	const int64_t hi = lo + a.per < a.count ? lo + a.per : a.count;
+	const int32_t c_lo = (int32_t)(lo / kWaves);
+	const int32_t c_hi = (int32_t)((hi + kWaves - 1) / kWaves);
+	int at = 0;
+	double acc = 0.0;
+
+	if (a.n_fix > 0) {
+		int len = a.n_fix;
+
+		/* the first entry not below c_lo (the same for every lane) */
+		while (len > 0) {
+			const int half = len / 2;
+
+			if (a.fix[at + half] < c_lo) {
+				at += half + 1;
+				len -= half + 1;
+			} else {
+				len = half;
+			}
+		}
+		for (; at < a.n_fix && a.fix[at] < c_hi; at++) {
+			const int64_t c = a.fix[at];
+			double x = (NT && c < a.sum.keep_from) ? chunk_sum_lane<true>(a.sum, c, tid)
+			    : chunk_sum_lane<false>(a.sum, c, tid);
+
+#pragma unroll
+			for (int off = 32; off > 0; off >>= 1)
+				x += __shfl_down(x, off, 64);
+			if ((tid & 63) == 0)
+				__hip_atomic_store(cells + c * kWaves + (tid >> 6),
+				    (unsigned long long)__double_as_longlong(x), __ATOMIC_RELAXED,
+				    __HIP_MEMORY_SCOPE_AGENT);
+		}
+		__syncthreads();
+	}
+	for (int64_t i0 = lo + tid; i0 < hi; i0 += (int64_t)kFoldAhead * kThreads) {
+		unsigned long long v[kFoldAhead];
+
+#pragma unroll
+		for (int k = 0; k < kFoldAhead; k++) {
+			const int64_t i = i0 + (int64_t)k * kThreads;
+
+			v[k] = i < hi ? __hip_atomic_load(cells + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+			    : 0ull;
+		}
+#pragma unroll
+		for (int k = 0; k < kFoldAhead; k++)
+			if (i0 + (int64_t)k * kThreads < hi)
+				acc += __longlong_as_double((long long)v[k]);
+	}
+	const double total = block_sum(acc, lds);
+
+	__syncthreads();		/* lds is used again below */
+	sumsq_finish(a.fin, total, lds, &last);
+	/* the lane that stored the state tells a host that is watching `stamp` (page-locked memory) */
+	if (last && a.stamp && tid == 0) {
+		__threadfence_system();
+		__hip_atomic_store(a.stamp, a.token, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+	}
+}
+
 /* ---- the update ---------------------------------------------------------- */
 
 struct UpdateArgs {
@@ -543,6 +765,8 @@ struct UpdateArgs {
 	uint32_t	uniform_flags;
 	int		vec_ok;
 	int		reverse;	/* walk the tiles from the last to the first */
+	const int32_t	*order;		/* not NULL: only the tiles order[0 .. turns), in that order (adam_update_kernel) */
+	int64_t		turns;
 	StepConsts	c;
 	double		grad_scale;
 	int		use_norm;	/* scale and skip come from *state, stored by the sum of squares */
@@ -570,7 +794,8 @@ template <int GT>
 __device__ __forceinline__ TileInfo tile_info(const UpdateArgs &a, int64_t turn, bool skip)
 {
 	TileInfo t;
-	const int64_t tile = a.reverse ? (a.n + kTile - 1) / kTile - 1 - turn : turn;
+	const int64_t tile = a.order ? (int64_t)a.order[turn]
+	    : a.reverse ? (a.n + kTile - 1) / kTile - 1 - turn : turn;
 
 	t.tile = tile;
 	t.base = tile * kTile;
@@ -593,7 +818,7 @@ template <int GT, int MT, int U, bool NT, bool DER>
 __global__ __launch_bounds__(kThreads) void adam_update_kernel(UpdateArgs a)
 {
 	const int tid = threadIdx.x;
-	const int64_t n_tiles = (a.n + kTile - 1) / kTile;
+	const int64_t n_tiles = a.order ? a.turns : (a.n + kTile - 1) / kTile;
 	double gs = a.grad_scale;
 	bool skip = false;
 
@@ -1420,6 +1645,7 @@ static int sumsq_launch(hipStream_t st, const Flat &f, double grad_scale, double
 */
 static const int kGuardDevices = 64;
 static std::atomic<int> g_fold_checked[kGuardDevices];
+static std::atomic<int> g_finish_checked[kGuardDevices];	/* chunk_finish_kernel: 0 not checked yet, 1 good, 2 use the separate kernels */
 static std::mutex g_fold_mu;
 static StepState *g_fold_host;		/* page-locked, two states */
 static int g_fold_runs;
@@ -1427,8 +1653,10 @@ static int g_fold_mismatches;
 
 static void fold_guard_reset(void)
 {
-	for (int i = 0; i < kGuardDevices; i++)
+	for (int i = 0; i < kGuardDevices; i++) {
 		g_fold_checked[i].store(0, std::memory_order_relaxed);
+		g_finish_checked[i].store(0, std::memory_order_relaxed);
+	}
 }
 
 void fold_guard_stats(int *runs, int *mismatches)
@@ -1498,6 +1726,171 @@ int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *parti
 	    && partials)
 		fold_guard(st, f, grad_scale, partials, fin);
 	return sumsq_launch(st, f, grad_scale, partials, n_partials, fin, sw().fold_fence);
+}
+
+int chunk_sums_count(int64_t n)
+{
+	const int64_t c = (n + SumsqChunk<kF32>::kElems - 1) / SumsqChunk<kF32>::kElems;
+
+	return (int)c;
+}
+
+int launch_chunk_sums(hipStream_t st, const float *x, int64_t n, double *part, const int32_t *list,
+	int n_list)
+{
+	ChunkSumArgs a;
+	const int64_t n_chunks = chunk_sums_count(n);
+	int64_t grid;
+
+	if (!x || n <= 0 || !part || (list && n_list <= 0))
+		return -1;
+	a.x = x;
+	a.n = n;
+	a.part = part;
+	a.list = list;
+	a.n_list = list ? n_list : 0;
+	a.vec_ok = aligned(x, 16) ? 1 : 0;
+	{
+		const int64_t keep = (int64_t)keep_mb() * (1 << 20) / SumsqChunk<kF32>::kBytes;
+
+		a.keep_from = n_chunks > keep ? n_chunks - keep : 0;
+	}
+	if (list) {
+		grid = n_list;
+	} else {
+		grid = (int64_t)cu_count() * (sw().sumsq_per_cu ? sw().sumsq_per_cu : 2);
+		if (grid > n_chunks)
+			grid = n_chunks;
+	}
+	if (grid < 1)
+		grid = 1;
+	if (nt_on())
+		hipLaunchKernelGGL((chunk_sums_kernel<true>), dim3((unsigned)grid), dim3(kThreads), 0, st, a);
+	else
+		hipLaunchKernelGGL((chunk_sums_kernel<false>), dim3((unsigned)grid), dim3(kThreads), 0, st, a);
+	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int launch_chunk_fold(hipStream_t st, const double *part, int64_t n, double *runs, StepState *state)
+{
+	const int64_t count = (int64_t)chunk_sums_count(n) * kWaves;
+	int64_t per = 2048;		/* partials per run: eight per lane */
+	int64_t n_runs;
+
+	if (!part || !runs || !state || n <= 0)
+		return -1;
+	while ((count + per - 1) / per > kChunkRuns)
+		per *= 2;
+	n_runs = (count + per - 1) / per;
+	hipLaunchKernelGGL(chunk_fold_kernel, dim3((unsigned)n_runs), dim3(kThreads), 0, st, part, count, per, runs);
+	hipLaunchKernelGGL(chunk_final_kernel, dim3(1), dim3(kThreads), 0, st, (const double *)runs, (int)n_runs,
+	    state);
+	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+/*
+** Self-check of chunk_finish_kernel, as for the sum of squares' second stage (fold_guard): the
+** first call on each device, and the first after the switches were read again, runs the merged
+** kernel and the three separate ones (which hand nothing over inside a launch) on the caller's
+** own flat, waits, and compares the two states bit for bit.  If they differ the process stays
+** with the separate kernels and says so once on stderr.
+*/
+
+static int chunk_finish_launch(hipStream_t st, const float *x, int64_t n, double *part, const int32_t *fix,
+	int n_fix, double *runs, unsigned int *ticket, StepState *state, unsigned long long *stamp,
+	unsigned long long token)
+{
+	static ChunkFinishArgs a;	/* 3 KiB: off the stack; calls are serialised by the caller */
+	const int64_t n_chunks = chunk_sums_count(n);
+	const int64_t keep = (int64_t)keep_mb() * (1 << 20) / SumsqChunk<kF32>::kBytes;
+	int64_t per = 2048;
+
+	a.count = n_chunks * kWaves;
+	while ((a.count + per - 1) / per > kChunkRuns)
+		per *= 2;
+	a.per = per;
+	a.sum.x = x;
+	a.sum.n = n;
+	a.sum.part = part;
+	a.sum.list = nullptr;
+	a.sum.n_list = 0;
+	a.sum.vec_ok = aligned(x, 16) ? 1 : 0;
+	a.sum.keep_from = n_chunks > keep ? n_chunks - keep : 0;
+	memset(&a.fin, 0, sizeof(a.fin));
+	a.fin.partials = runs;
+	a.fin.ticket = ticket;
+	a.fin.grad_scale = 1.0;
+	a.fin.state = state;
+	a.fin.fence = sw().fold_fence;
+	a.stamp = stamp;
+	a.token = token;
+	a.n_fix = n_fix;
+	if (n_fix > 0)
+		memcpy(a.fix, fix, (size_t)n_fix * sizeof(int32_t));
+	const unsigned grid = (unsigned)((a.count + per - 1) / per);
+
+	if (nt_on())
+		hipLaunchKernelGGL((chunk_finish_kernel<true>), dim3(grid), dim3(kThreads), 0, st, a);
+	else
+		hipLaunchKernelGGL((chunk_finish_kernel<false>), dim3(grid), dim3(kThreads), 0, st, a);
+	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+static int chunk_finish_apart(hipStream_t st, const float *x, int64_t n, double *part, const int32_t *fix_dev,
+	int n_fix, double *runs, StepState *state)
+{
+	if (n_fix > 0 && launch_chunk_sums(st, x, n, part, fix_dev, n_fix) != 0)
+		return -1;
+	return launch_chunk_fold(st, part, n, runs, state);
+}
+
+int launch_chunk_finish(hipStream_t st, const float *x, int64_t n, double *part, const int32_t *fix,
+	const int32_t *fix_dev, int n_fix, double *runs, unsigned int *ticket, StepState *state,
+	unsigned long long *stamp, unsigned long long token)
+{
+	int dev = -1;
+	int how;
+
+	if (!x || n <= 0 || !part || !runs || !state || n_fix < 0 || (n_fix > 0 && (!fix || !fix_dev)))
+		return -1;
+	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kGuardDevices) {
+		(void)hipGetLastError();
+		dev = -1;
+	}
+	how = (dev < 0 || !ticket || !aligned(ticket, 128) || n_fix > kFixMax) ? 2
+	    : g_finish_checked[dev].load(std::memory_order_acquire);
+	if (how == 0) {
+		hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+		std::lock_guard<std::mutex> lk(g_fold_mu);
+
+		if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone
+		    || (!g_fold_host && hipHostMalloc((void **)&g_fold_host, 2 * sizeof(StepState),
+		    hipHostMallocPortable) != hipSuccess)) {
+			(void)hipGetLastError();
+			how = 2;	/* this call only: the check is put off */
+		} else {
+			memset(g_fold_host, 0xff, 2 * sizeof(StepState));
+			if (chunk_finish_launch(st, x, n, part, fix, n_fix, runs, ticket, g_fold_host, nullptr, 0) != 0
+			    || chunk_finish_apart(st, x, n, part, fix_dev, n_fix, runs, g_fold_host + 1) != 0
+			    || hipStreamSynchronize(st) != hipSuccess) {
+				(void)hipGetLastError();
+				return -1;
+			}
+			g_fold_runs++;
+			how = 1;
+			if (memcmp(&g_fold_host[0], &g_fold_host[1], sizeof(StepState)) != 0) {
+				g_fold_mismatches++;
+				how = 2;
+				fprintf(stderr, "[anni] sum of squares of a flat: the merged last stage and the separate "
+				    "kernels disagree on this device (sum %.17g against %.17g); using the separate "
+				    "kernels from now on\n", g_fold_host[0].sumsq, g_fold_host[1].sumsq);
+			}
+			g_finish_checked[dev].store(how, std::memory_order_release);
+		}
+	}
+	if (how == 1)
+		return chunk_finish_launch(st, x, n, part, fix, n_fix, runs, ticket, state, stamp, token);
+	return chunk_finish_apart(st, x, n, part, fix_dev, n_fix, runs, state) == 0 ? 1 : -1;
 }
 
 #ifndef ANNI_UPDATE_UNROLL
@@ -1591,8 +1984,8 @@ static int check_derived(const Flat &f)
 	return 0;
 }
 
-int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double grad_scale,
-	const NormIn &norm)
+static int update_go(hipStream_t st, const Flat &f, const StepConsts &c, double grad_scale,
+	const NormIn &norm, const int32_t *order, int64_t turns)
 {
 	UpdateArgs a;
 	int grid;
@@ -1602,6 +1995,16 @@ int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double gra
 	if (norm.use_norm && !norm.state)
 		return -1;
 	grid = balanced_grid(f.n, 1);
+	if (order) {
+		const bool narrow = f.grad_type != kF32 || f.moment_type != kF32;
+
+		/* the software-pipelined kernels walk the flat their own way */
+		if (turns < 1 || turns > (f.n + kTile - 1) / kTile || pipe_level() >= (narrow ? 1 : 2))
+			return -1;
+		grid = balanced_grid(turns * kTile, 1);
+	}
+	a.order = order;
+	a.turns = order ? turns : 0;
 	a.p = f.p;
 	a.g = f.g;
 	a.m = f.m;
@@ -1639,6 +2042,25 @@ int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double gra
 			update_launch<kFP8, kBF16>(st, grid, a);
 	}
 	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int launch_update(hipStream_t st, const Flat &f, const StepConsts &c, double grad_scale,
+	const NormIn &norm)
+{
+	return update_go(st, f, c, grad_scale, norm, nullptr, 0);
+}
+
+int update_walks_backwards(void)
+{
+	return reverse_on() ? 1 : 0;
+}
+
+int launch_update_tiles(hipStream_t st, const Flat &f, const StepConsts &c, double grad_scale,
+	const NormIn &norm, const int32_t *order, int64_t turns)
+{
+	if (!order)
+		return -1;
+	return update_go(st, f, c, grad_scale, norm, order, turns);
 }
 
 static int helper_grid(int64_t work_items)

@@ -21,8 +21,12 @@ extern "C" {
 int	anni_hook_step_events(anni_adam *opt, double lr, double grad_scale, void *const events[4]);
 /* Reads the ANNI_* tuning switches from the environment again; the next sum of squares re-runs its self-check. */
 void	anni_hook_reload_switches(void);
-/* How often the self-check of the sum of squares' second stage has run in this process, and how often its two forms disagreed. */
-void	anni_hook_fold_guard_stats(int *runs, int *mismatches);
+/*
+** Counters the library keeps for the record, by name; -1 for a name it does not know:
+**   "fold_guard_runs", "fold_guard_mismatches"   the self-check of the arena's sum of squares
+**   "early_sum_used", "early_sum_dropped"        gpu_grad_sumsq's sum begun early, taken / thrown away
+*/
+long	anni_hook_counter(const char *name);
 
 #ifdef __cplusplus
 }

@@ -36,6 +36,11 @@ bool		release_idle_pools(void);
 */
 hipError_t	device_alloc(void **p, size_t nbytes);
 
+/* How often the sum of squares begun early (gpu_backend.hip) was used by the call that followed, and how often dropped. */
+void		early_sum_stats(long *used, long *dropped);
+/* Steps whose small read-backs were served by a split update (gpu_backend.hip, "the vectors first"), and how many read-backs. */
+void		vectors_first_stats(long *steps, long *served);
+
 /*
 ** ANN_OP_PROF=1 (num/gpu_cuda.cu:3205-3409): an event pair around an operation of the optimizer
 ** step, summed per kind and printed by gpu_op_prof_dump.  prof_begin records the first event on

@@ -210,7 +210,28 @@ void anni_gpu_reload_switches(void)
 
 int anni_fold_guard_stats(int *runs, int *mismatches)
 {
-	anni_hook_fold_guard_stats(runs, mismatches);
+	if (runs)
+		*runs = (int)anni_hook_counter("fold_guard_runs");
+	if (mismatches)
+		*mismatches = (int)anni_hook_counter("fold_guard_mismatches");
+	return 0;
+}
+
+int anni_early_sum_stats(long *used, long *dropped)
+{
+	if (used)
+		*used = anni_hook_counter("early_sum_used");
+	if (dropped)
+		*dropped = anni_hook_counter("early_sum_dropped");
+	return 0;
+}
+
+int anni_vectors_first_stats(long *steps, long *served)
+{
+	if (steps)
+		*steps = anni_hook_counter("vectors_first_steps");
+	if (served)
+		*served = anni_hook_counter("vectors_first_served");
 	return 0;
 }
 

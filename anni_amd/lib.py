@@ -143,6 +143,8 @@ _BENCH_PROTOS = {
                                        C.c_float, C.c_float]),
     "anni_copy_bytes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "anni_fold_guard_stats": (C.c_int, [C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "anni_early_sum_stats": (C.c_int, [C.POINTER(C.c_long), C.POINTER(C.c_long)]),
+    "anni_vectors_first_stats": (C.c_int, [C.POINTER(C.c_long), C.POINTER(C.c_long)]),
 }
 
 _lib = None

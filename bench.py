@@ -358,6 +358,8 @@ def reference_caller_leg(L, size="185m", call_trace=False):
         make = lambda: ob.RefModelOnBackend(100000, beta2=0.95, weight_decay=0.1, grad_clip=1.0,
                                             backend="hip555m" + suffix, tied=True)
     L.gpu_set_compute_prec(1)
+    used0, dropped0 = C.c_long(0), C.c_long(0)
+    L.anni_early_sum_stats(C.byref(used0), C.byref(dropped0))
     M = make()
     n = M.n
     vec_bytes = 4 * sum(cnt for _off, cnt, is_mat in M.segs() if not is_mat)
@@ -365,7 +367,7 @@ def reference_caller_leg(L, size="185m", call_trace=False):
     g = rng.standard_normal(n, dtype=np.float32) * np.float32(1e-3)
     unit = 1.0 / (math.sqrt(n) * 1e-3)
     times = []
-    last = 9
+    last = 13
     for t in range(1, last + 1):
         M.set_grads(g)
         L.gpu_device_sync()
@@ -378,6 +380,8 @@ def reference_caller_leg(L, size="185m", call_trace=False):
             ob.gputrace().gputrace_stop()
     n_segs = M.n_segs
     events = ob.gputrace_events() if call_trace else None
+    used, dropped = C.c_long(0), C.c_long(0)
+    L.anni_early_sum_stats(C.byref(used), C.byref(dropped))
     M.close()
     L.gpu_set_compute_prec(0)
     L.gpu_adam_set_weight_decay(0.0)
@@ -389,7 +393,10 @@ def reference_caller_leg(L, size="185m", call_trace=False):
            "ms_per_step": round(ms, 3), "min_ms": round(min(times[1:]), 3),
            "first_step_ms_with_arena_init": round(times[0], 1),
            "GBps_algorithmic": round(n * 38 / ms / 1e6, 1),
-           "frac": round(n * 38 / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+           "frac": round(n * 38 / ms / 1e6 / HBM_PEAK_GBPS, 4),
+           "steps": last,
+           "sums_begun_at_the_first_upload_and_used": used.value - used0.value,
+           "sums_begun_early_and_dropped": dropped.value - dropped0.value}
     if events:
         out["call_trace_of_the_last_step"] = call_timeline(events, times[-1])
     return out

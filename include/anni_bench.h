@@ -49,6 +49,20 @@ void	anni_gpu_reload_switches(void);
 ** process has gone over to the conservative form and said so on stderr).  Returns 0.
 */
 int	anni_fold_guard_stats(int *runs, int *mismatches);
+/*
+** gpu_grad_sumsq may begin its sum before it is called, when the caller has shown the pattern of
+** lang/lm_adam.c twice in a row (small uploads of vectors, then the sum of the same flat): how
+** often such an early sum was used by the call that followed, and how often it had to be thrown
+** away because something else had gone onto the stream or another flat was named.  Returns 0.
+*/
+int	anni_early_sum_stats(long *used, long *dropped);
+/*
+** gpu_adam_step_dev_bf16 may update the tiles that hold the caller's bias / LayerNorm vectors in a
+** launch of their own and copy those vectors out ahead of the rest, when the caller has read the
+** same list of small ranges back after two updates in a row (lang/lm_adam.c:407-413): the steps
+** in which read-backs were served that way, and how many read-backs.  Returns 0.
+*/
+int	anni_vectors_first_stats(long *steps, long *served);
 
 #ifdef __cplusplus
 }

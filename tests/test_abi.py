@@ -41,7 +41,7 @@ def test_every_declared_symbol_is_exported_and_nothing_else():
     hooks = declared_in(os.path.join(ROOT, "anni_amd", "csrc", "anni_hooks.h"))
     bench = declared_in(os.path.join(inc, "anni_bench.h")) - product
     assert len([s for s in product if s.startswith("gpu_")]) == 99          # the whole of num/gpu.h
-    assert hooks == {"anni_hook_step_events", "anni_hook_reload_switches", "anni_hook_fold_guard_stats"}
+    assert hooks == {"anni_hook_step_events", "anni_hook_reload_switches", "anni_hook_counter"}
     assert exported_by(lib.SO_PATH) == product | hooks
     assert exported_by(lib.BENCH_SO_PATH) == bench
     assert set(glob.glob(os.path.join(inc, "*.h"))) == {os.path.join(inc, h) for h in
