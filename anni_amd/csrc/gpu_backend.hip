@@ -148,6 +148,20 @@ struct Delivery {
 };
 static Delivery g_deliver[kDescSlots];	/* gathered D2H data waiting for a synchronisation */
 static int g_deliver_n;
+/*
+** The device ranges of the uploads that wait for the next launch, sorted, none overlapping another.
+** The pieces of one launch are copied in no particular order, so an upload that overlaps one of them
+** must not share their launch: the caller's order (the later copy wins) is kept by the launch boundary.
+*/
+struct UpRange {
+	uintptr_t	lo, hi;
+};
+static std::vector<UpRange> g_up_pending;
+static bool up_before(const UpRange &a, const UpRange &b)
+{
+	return a.lo < b.lo;
+}
+static const size_t kUpPendingMax = 512;	/* more than that waiting: launch, so that the list stays short */
 
 /*
 ** One workgroup per piece.  The staging side of every copy is placed at the same offset from
@@ -240,6 +254,7 @@ static void batch_flush_locked(void)
 	g_batch_first = g_desc_used;
 	g_batch_bytes = 0;
 	g_batch_dir = 0;
+	g_up_pending.clear();
 }
 
 /* After the stream has drained: hand gathered data to its host destinations, recycle the rings.  g_mu held. */
@@ -272,6 +287,13 @@ static bool batch_add_locked(int dir, void *dev, void *host, size_t nbytes)
 	if (g_batch_dir != 0 && g_batch_dir != dir)
 		batch_flush_locked();
 	if (dir == 1) {
+		const UpRange r = {(uintptr_t)dev, (uintptr_t)dev + nbytes};
+		const auto nx = std::lower_bound(g_up_pending.begin(), g_up_pending.end(), r, up_before);
+
+		if ((nx != g_up_pending.end() && nx->lo < r.hi)
+		    || (nx != g_up_pending.begin() && (nx - 1)->hi > r.lo)
+		    || g_up_pending.size() >= kUpPendingMax)
+			batch_flush_locked();		/* what it overlaps goes first, in a launch of its own */
 		vf_on_small_h2d_locked();
 		early_sum_on_small_h2d_locked(dev, nbytes);	/* may put the sum of the gradient flat on the stream first */
 	}
@@ -291,7 +313,10 @@ static bool batch_add_locked(int dir, void *dev, void *host, size_t nbytes)
 		g_desc_used++;
 	}
 	if (dir == 1) {
+		const UpRange r = {(uintptr_t)dev, (uintptr_t)dev + nbytes};
+
 		memcpy(g_stage + at, host, nbytes);
+		g_up_pending.insert(std::lower_bound(g_up_pending.begin(), g_up_pending.end(), r, up_before), r);
 	} else {
 		g_deliver[g_deliver_n].host = host;
 		g_deliver[g_deliver_n].stage_off = at;

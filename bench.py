@@ -360,6 +360,8 @@ def reference_caller_leg(L, size="185m", call_trace=False):
     L.gpu_set_compute_prec(1)
     used0, dropped0 = C.c_long(0), C.c_long(0)
     L.anni_early_sum_stats(C.byref(used0), C.byref(dropped0))
+    vsteps0, vserved0 = C.c_long(0), C.c_long(0)
+    L.anni_vectors_first_stats(C.byref(vsteps0), C.byref(vserved0))
     M = make()
     n = M.n
     vec_bytes = 4 * sum(cnt for _off, cnt, is_mat in M.segs() if not is_mat)
@@ -382,6 +384,8 @@ def reference_caller_leg(L, size="185m", call_trace=False):
     events = ob.gputrace_events() if call_trace else None
     used, dropped = C.c_long(0), C.c_long(0)
     L.anni_early_sum_stats(C.byref(used), C.byref(dropped))
+    vsteps, vserved = C.c_long(0), C.c_long(0)
+    L.anni_vectors_first_stats(C.byref(vsteps), C.byref(vserved))
     M.close()
     L.gpu_set_compute_prec(0)
     L.gpu_adam_set_weight_decay(0.0)
@@ -392,11 +396,14 @@ def reference_caller_leg(L, size="185m", call_trace=False):
            "params": n, "segments": n_segs, "host_vector_bytes": vec_bytes,
            "ms_per_step": round(ms, 3), "min_ms": round(min(times[1:]), 3),
            "first_step_ms_with_arena_init": round(times[0], 1),
+           "ms_of_steps_2_to_4_while_the_callers_pattern_is_learned": [round(x, 3) for x in times[1:4]],
            "GBps_algorithmic": round(n * 38 / ms / 1e6, 1),
            "frac": round(n * 38 / ms / 1e6 / HBM_PEAK_GBPS, 4),
            "steps": last,
            "sums_begun_at_the_first_upload_and_used": used.value - used0.value,
-           "sums_begun_early_and_dropped": dropped.value - dropped0.value}
+           "sums_begun_early_and_dropped": dropped.value - dropped0.value,
+           "steps_with_the_vectors_updated_and_read_back_first": vsteps.value - vsteps0.value,
+           "read_backs_served_that_way": vserved.value - vserved0.value}
     if events:
         out["call_trace_of_the_last_step"] = call_timeline(events, times[-1])
     return out
@@ -423,12 +430,15 @@ def call_timeline(ev, wall_ms):
                                for nm, (c, us, by) in sorted(per.items(), key=lambda kv: -kv[1][1]) if us >= 0.05},
         "callers_own_time_between_calls_us": r(sum(ev[i + 1][1] - ev[i][2] for i in range(len(ev) - 1))),
         "phases_us": {
-            "gather: step start .. gpu_grad_sumsq called (the caller stages its vectors; device idle "
-            "but for the copy pieces)": r(ev[i_ss][1] - base),
-            "gpu_grad_sumsq (last copy piece, sum of squares, wait, read-back)": r(ev[i_ss][2] - ev[i_ss][1]),
-            "norm on the host .. update launched": r(ev[i_st][2] - ev[i_ss][2]),
-            "scatter calls (queued behind the update)": r(ev[i_sy][1] - ev[i_st][2]),
-            "gpu_stream_sync (rest of the update, copy-back kernel, wait, hand-over to the caller's vectors)":
+            "gather: step start .. gpu_grad_sumsq called (the caller stages its vectors; on the device "
+            "the copy pieces and, once the pattern is learned, the sum begun at the first upload)":
+                r(ev[i_ss][1] - base),
+            "gpu_grad_sumsq (last copy piece, rest of the sum, its last stage, result read from "
+            "page-locked memory)": r(ev[i_ss][2] - ev[i_ss][1]),
+            "norm on the host .. update launched (in two parts once the read-backs are learned)":
+                r(ev[i_st][2] - ev[i_ss][2]),
+            "the caller's read-back calls": r(ev[i_sy][1] - ev[i_st][2]),
+            "gpu_stream_sync (the vectors handed over while the update runs, then the wait for it)":
                 r(ev[i_sy][2] - ev[i_sy][1]),
             "after": r(ev[-1][2] - ev[i_sy][2])},
         "calls_over_10us": [{"entry": nm, "at_us": r(a - base), "us": r(b - a), "bytes": by}

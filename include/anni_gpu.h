@@ -17,6 +17,17 @@
 ** and kernel is issued on one in-order compute stream; gpu_memcpy_d2h blocks.
 ** Buffers are owned by the caller (gpu_malloc / gpu_free); the backend only
 ** borrows the registered twin flat.
+**
+** Threads: gpu_grad_sumsq and gpu_adam_step_dev_bf16 keep one result slot, one
+** set of partial sums and one set of ticket words per process, as the reference's
+** do (static s_acc, num/gpu_cuda.cu:8485-8486): they are for ONE thread on the
+** library's one compute stream.  The memory functions may be called from any thread.
+**
+** Order of completion is the order of the calls, always.  Within that contract the
+** library may begin work before it is asked for, on a second stream of its own, when
+** a caller has shown the call order of lang/lm_adam.c:452-515 twice in a row (small
+** uploads, the sum of squares, the update, small read-backs, a synchronisation); see
+** gpu_grad_sumsq and gpu_adam_step_dev_bf16 below.  Results do not depend on it.
 */
 #ifndef ANNI_GPU_H__
 #define ANNI_GPU_H__
@@ -123,7 +134,15 @@ int	gpu_mat_col_sum_add(ann_real *db_host, const ann_real *x, int rows, int cols
 void	gpu_adam_set_weight_decay(double wd);
 /*
 ** num/gpu.h:123 -- *out = sum of d_x[i]^2 over n device floats, accumulated in
-** double in a fixed order (run-to-run deterministic).  Implies a stream sync.
+** double in a fixed order that depends on n alone (run-to-run deterministic).
+** Everything put on the compute stream before the call has completed when it
+** returns.  -1 also when another thread's call is between its launch and its
+** read-back (one result slot per process; the caller takes its CPU path).
+** Once the caller has twice in a row synchronised, made nothing but small uploads
+** into this flat and the registered parameter flat, and then asked for this sum,
+** the sum over the chunks those uploads do not touch is begun at the first such
+** upload of the next step; the call then only adds the chunks written since.
+** Same bits either way.  ANNI_EARLY_SUM=0 switches that off.
 */
 int	gpu_grad_sumsq(const ann_real *d_x, int n, double *out);
 /*
@@ -134,6 +153,11 @@ int	gpu_grad_sumsq(const ann_real *d_x, int n, double *out);
 ** NULL pointer, n <= 0, lr <= 0, t < 1, 1-beta^t <= 0 or no device.
 ** The arithmetic follows the reference's host loop (lang/lm_adam.c:587-598) in
 ** double, so results equal the CPU path bit for bit for the same grad_scale.
+** Once the caller has read the same list of small ranges of d_param back
+** (gpu_memcpy_d2h_async) after two steps in a row, the tiles holding those ranges
+** are updated by a launch of their own and copied out ahead of the rest, so that
+** gpu_stream_sync can hand them over while the large launch is still running; only
+** when the compute stream is idle at the call.  ANNI_VECTORS_FIRST=0 switches that off.
 */
 int	gpu_adam_step_dev_bf16(ann_real *d_param, void *d_param_bf16, ann_real *d_grad,
 		ann_real *d_m, ann_real *d_v, int n, double lr, double beta1,

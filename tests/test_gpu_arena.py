@@ -730,3 +730,34 @@ def test_gnorm_every_alone_computes_and_prints_the_norm(gpu):
     assert len(norms) == 4 and all(abs(float(x[2]) - want) < 1e-9 * want and x[3] == "0" for x in norms)
     said = [ln for ln in r.stderr.splitlines() if ln.startswith("[adam] step ")]
     assert said == ["[adam] step 2 grad norm %.4g" % want, "[adam] step 4 grad norm %.4g" % want], r.stderr
+
+
+def test_op_prof_times_the_arena_steps_launches(gpu):
+    """ANN_OP_PROF=1 (num/gpu_cuda.cu:3205-3409, lang/lm_adam.c:541): every launch of the optimizer
+    step is bracketed by an event pair and the table is printed after each step, on the arena path as
+    on the flat entry points (the switch is read once per process: a child)."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    child = (
+        "import sys; sys.path.insert(0, %r)\n"
+        "import numpy as np\n"
+        "from anni_amd.lm_adam import LmAdam\n"
+        "opt = LmAdam([(300000, 3), (77, 0)], grad_clip=1.0)\n"
+        "for s in range(3):\n"
+        "    opt.upload('grad', np.full(opt.n, 0.5, np.float32))\n"
+        "    opt.step_scaled(1e-3)\n"
+        "    opt.sync_stats()\n"
+    ) % root
+    env = dict(os.environ, ANN_OP_PROF="1")
+    r = subprocess.run([sys.executable, "-c", child], env=env, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr[-1500:]
+    rows = [ln.split() for ln in r.stderr.splitlines() if ln.startswith("[op-prof] ")]
+    per = {}
+    for w in rows:                                        # [op-prof] name ms "ms" calls "calls"
+        per.setdefault(w[1], []).append((float(w[2]), int(w[4])))
+    assert set(per) == {"grad_sumsq", "adam_step"}, r.stderr
+    for name, got in per.items():
+        assert sum(c for _ms, c in got) == 3, (name, got)
+        assert all(0.0 < ms < 50.0 for ms, _c in got), (name, got)

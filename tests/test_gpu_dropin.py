@@ -531,6 +531,41 @@ def test_small_copies_are_batched_in_order(gpu):
     assert not d.download(np.uint8, 4096).any()
 
 
+def test_small_uploads_that_overlap_keep_the_callers_order(gpu):
+    """The pieces of one batch are copied in no particular order, so an upload that overlaps one
+    still waiting must go into a later launch: as with separate copies, the later one wins.
+    Checked with no synchronisation between the uploads: the same bytes many times, ranges that
+    overlap in part, neighbours that only touch (which may share a launch), and more uploads
+    waiting than the list of waiting ranges holds."""
+    from anni_amd.lm_adam import DeviceBuffer
+    rng = np.random.default_rng(8)
+    size = 1 << 20
+    d = DeviceBuffer(size)
+    want = np.zeros(size, np.uint8)
+    assert gpu.gpu_memset(d.ptr, 0, size) == 0
+    keep = []                                            # the host buffers may be reused, but keep them anyway
+
+    def up(off, values):
+        a = np.ascontiguousarray(values, dtype=np.uint8)
+        keep.append(a)
+        want[off:off + a.size] = a
+        assert gpu.gpu_memcpy_h2d(d.ptr + off, a.ctypes.data, a.size) == 0
+    for k in range(300):                                 # the same four bytes, 300 times
+        up(1000, np.full(4, k % 251, np.uint8))
+    for k in range(200):                                 # sliding windows, each overlapping the last
+        up(5000 + 37 * k, rng.integers(0, 255, 100, dtype=np.uint8))
+    for k in range(100):                                 # neighbours that only touch
+        up(40000 + 64 * k, np.full(64, k, np.uint8))
+    for k in range(700):                                 # many disjoint bytes, then all of them again
+        up(100000 + 16 * k, [k % 256])
+    for k in range(700):
+        up(100000 + 16 * k, [(k * 7 + 1) % 256])
+    up(0, rng.integers(0, 255, 300000, dtype=np.uint8))  # a large one over everything so far ...
+    up(999, np.full(10, 77, np.uint8))                   # ... and a small one on top of it
+    assert (d.download(np.uint8, size) == want).all()
+    d.free()
+
+
 def test_batched_copies_and_the_librarys_own_syncs(gpu):
     """A small gpu_memcpy_d2h_async is complete after ANY synchronising call of the library, the
     arena's included, and anni_gpu_flush puts a pending small upload on the stream for work the
