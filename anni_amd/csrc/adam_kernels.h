@@ -149,17 +149,19 @@ int	launch_update_tiles(hipStream_t st, const Flat &f, const StepConsts &c, doub
 		const NormIn &norm, const int32_t *order, int64_t turns);
 /*
 ** The sum of squares of a float flat in separable steps (the flat entry point gpu_grad_sumsq):
-** launch_chunk_sums writes kWaves partial sums for every 16 KiB chunk of x (list == NULL) or for
-** the n_list chunks named in `list` (device-readable memory) into part[chunk * kWaves ..];
-** launch_chunk_fold adds all chunk_sums_count(n) * kWaves partials in index order, through at
-** most kChunkRuns intermediate sums in `runs`, and stores {sum, sqrt(sum), 1, 0, 0} into *state.
+** launch_chunk_sums writes one partial sum for every 16 KiB chunk of x (list == NULL) or for
+** the n_list chunks named in `list` (device-readable memory) into part[chunk];
+** launch_chunk_fold adds all chunk_sums_count(n) partials in index order, through at most
+** kChunkRuns intermediate sums (of kChunkPer partials or a power of two times that) in `runs`,
+** and stores {sum, sqrt(sum), 1, 0, 0} into *state.
 ** The sum is a function of x alone: partials recomputed for some chunks after their elements
 ** changed give the bits a pass over the whole flat would.
 */
 constexpr int kChunkRuns = 1024;
+constexpr int kChunkPer = 512;		/* two partials per lane of the workgroup that folds a run */
 int	chunk_sums_count(int64_t n);
 int	launch_chunk_sums(hipStream_t st, const float *x, int64_t n, double *part, const int32_t *list,
-		int n_list);
+		int n_list, int beside);	/* beside != 0: other kernels run at the same time, leave them room */
 int	launch_chunk_fold(hipStream_t st, const double *part, int64_t n, double *runs, StepState *state);
 /*
 ** The end of the sum in one launch: the partials of the n_fix chunks in `fix` (rising, no chunk

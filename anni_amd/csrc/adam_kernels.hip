@@ -528,12 +528,12 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(SumsqArgs a)
 	sumsq_finish(a, total, lds, &last);
 }
 
-/* ---- sum of squares of a float flat, one partial per wavefront and chunk --------------- */
+/* ---- sum of squares of a float flat, one partial per chunk ------------------------------ */
 
 /*
 ** The flat entry point (gpu_grad_sumsq) sums in two steps that can be taken apart: first every
-** 16 KiB chunk of the flat gets four partial sums, one per wavefront of the workgroup that read
-** it (shuffles only, no barrier), then the partials are folded in index order -- chunk_fold_kernel
+** 16 KiB chunk of the flat gets a partial sum, computed by one wavefront alone (shuffles only, no
+** barrier, nothing shared), then the partials are folded in index order -- chunk_fold_kernel
 ** over contiguous runs, chunk_final_kernel over the runs' sums.  The result is a pure function of
 ** the flat: it does not depend on the grid, and recomputing the partials of some chunks after
 ** their elements changed gives bit for bit what a pass over the whole flat gives.  That is what
@@ -543,30 +543,39 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(SumsqArgs a)
 struct ChunkSumArgs {
 	const float	*x;
 	int64_t		n;
-	double		*part;		/* kWaves per chunk */
-	const int32_t	*list;		/* NULL: every chunk; else the chunks to (re)compute, one per workgroup */
+	double		*part;		/* one per chunk */
+	const int32_t	*list;		/* NULL: every chunk; else the chunks to (re)compute, one per wavefront */
 	int		n_list;
 	int		vec_ok;
 	int64_t		keep_from;	/* chunks from here on are read with ordinary (cacheable) loads */
 };
 
+/*
+** The sum of the squares of chunk c, by ONE wavefront: lane l reads the 16 bytes at l, l + 64, ...,
+** l + 960 (in units of 16 bytes: sixteen loads, 1 KiB of the chunk per load instruction, all in
+** flight together), adds the squares of each of the four floats of a load to a chain of its own,
+** and the wavefront folds by shuffles.  The result is in lane 0.  A chunk that runs past the flat,
+** or a flat that is not 16-byte aligned, goes element by element.
+*/
 template <bool NT>
-__device__ __forceinline__ double chunk_sum_lane(const ChunkSumArgs &a, int64_t c, int tid)
+__device__ __forceinline__ double chunk_sum_wave(const ChunkSumArgs &a, int64_t c, int lane)
 {
 	typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 	constexpr int64_t kElems = SumsqChunk<kF32>::kElems;
+	constexpr int kLoads = (int)(SumsqChunk<kF32>::kBytes / (64 * 16));
 	const int64_t base = c * kElems;
 	double acc[4] = {0.0, 0.0, 0.0, 0.0};
+	double x;
 
 	if (a.vec_ok && base + kElems <= a.n) {
-		const u32x4 *src = (const u32x4 *)(a.x + base) + tid;
-		u32x4 W[4];
+		const u32x4 *src = (const u32x4 *)(a.x + base) + lane;
+		u32x4 W[kLoads];
 
 #pragma unroll
-		for (int u = 0; u < 4; u++)
-			W[u] = ld<NT>(src + u * kThreads);
+		for (int u = 0; u < kLoads; u++)
+			W[u] = ld<NT>(src + u * 64);
 #pragma unroll
-		for (int u = 0; u < 4; u++) {
+		for (int u = 0; u < kLoads; u++) {
 #pragma unroll
 			for (int k = 0; k < 4; k++) {
 				const double v = (double)__uint_as_float(W[u][k]);
@@ -577,41 +586,52 @@ __device__ __forceinline__ double chunk_sum_lane(const ChunkSumArgs &a, int64_t 
 	} else {
 		const int64_t end = base + kElems < a.n ? base + kElems : a.n;
 
-		for (int64_t i = base + tid; i < end; i += kThreads) {
+		for (int64_t i = base + lane; i < end; i += 64) {
 			const double v = (double)a.x[i];
 
 			acc[0] += v * v;
 		}
 	}
-	return (acc[0] + acc[1]) + (acc[2] + acc[3]);
+	x = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+#pragma unroll
+	for (int off = 32; off > 0; off >>= 1)
+		x += __shfl_down(x, off, 64);
+	return x;
 }
 
+/*
+** Wavefront w of workgroup b takes the chunks 4 b + w, 4 (b + gridDim.x) + w, ...: a workgroup
+** walks the flat in pieces of 64 KiB, each wavefront a contiguous quarter, and no wavefront waits
+** for another.  With a list, wavefront 4 b + w takes the chunk list[4 b + w].
+*/
 template <bool NT>
 __global__ __launch_bounds__(kThreads) void chunk_sums_kernel(ChunkSumArgs a)
 {
 	constexpr int64_t kElems = SumsqChunk<kF32>::kElems;
-	const int tid = threadIdx.x;
+	const int lane = threadIdx.x & 63;
+	const int64_t wave = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);
 	const int64_t n_chunks = (a.n + kElems - 1) / kElems;
-	const int64_t first = a.list ? 0 : blockIdx.x;
-	const int64_t step = a.list ? 1 : gridDim.x;
-	const int64_t stop = a.list ? 1 : n_chunks;
 
-	/*
-	** (Keeping the loads of a workgroup's next chunk in flight while it folds the current one was
-	** measured no faster: 0.389 against 0.381 ms per call at 555M.)
-	*/
-	for (int64_t k = first; k < stop; k += step) {
-		const int64_t c = a.list ? (int64_t)a.list[blockIdx.x] : k;
-		double x;
+	if (a.list) {
+		if (wave < a.n_list) {
+			const int64_t c = (int64_t)a.list[wave];
 
-		if (c < 0 || c >= n_chunks)
-			continue;
-		x = (NT && c < a.keep_from) ? chunk_sum_lane<true>(a, c, tid) : chunk_sum_lane<false>(a, c, tid);
-#pragma unroll
-		for (int off = 32; off > 0; off >>= 1)
-			x += __shfl_down(x, off, 64);
-		if ((tid & 63) == 0)
-			a.part[c * kWaves + (tid >> 6)] = x;
+			if (c >= 0 && c < n_chunks) {
+				const double x = (NT && c < a.keep_from) ? chunk_sum_wave<true>(a, c, lane)
+				    : chunk_sum_wave<false>(a, c, lane);
+
+				if (lane == 0)
+					a.part[c] = x;
+			}
+		}
+		return;
+	}
+	for (int64_t c = wave; c < n_chunks; c += (int64_t)gridDim.x * kWaves) {
+		const double x = (NT && c < a.keep_from) ? chunk_sum_wave<true>(a, c, lane)
+		    : chunk_sum_wave<false>(a, c, lane);
+
+		if (lane == 0)
+			a.part[c] = x;
 	}
 }
 
@@ -673,7 +693,7 @@ constexpr int kFixMax = 768;
 struct ChunkFinishArgs {
 	ChunkSumArgs	sum;		/* list unused */
 	int64_t		count;		/* partials in all */
-	int64_t		per;		/* partials per run, a multiple of kWaves */
+	int64_t		per;		/* partials per run */
 	SumsqArgs	fin;		/* partials = the runs' sums, ticket, state, fence */
 	unsigned long long	*stamp;	/* may be NULL: receives `token` once the state is stored */
 	unsigned long long	token;
@@ -686,41 +706,46 @@ __global__ __launch_bounds__(kThreads) void chunk_finish_kernel(ChunkFinishArgs 
 {
 	__shared__ double lds[4];
 	__shared__ int last;
+	__shared__ int32_t fix_s[kFixMax];
 	unsigned long long *cells = (unsigned long long *)a.sum.part;
 	const int tid = threadIdx.x;
 	const int64_t lo = (int64_t)blockIdx.x * a.per;
 	const int64_t hi = lo + a.per < a.count ? lo + a.per : a.count;
-	const int32_t c_lo = (int32_t)(lo / kWaves);
-	const int32_t c_hi = (int32_t)((hi + kWaves - 1) / kWaves);
+	const int32_t c_lo = (int32_t)lo;	/* one partial per chunk */
+	const int32_t c_hi = (int32_t)hi;
 	int at = 0;
 	double acc = 0.0;
 
 	if (a.n_fix > 0) {
 		int len = a.n_fix;
 
+		/*
+		** The list into LDS first, all lanes at once: the kernel's arguments may lie in host
+		** memory, where every step of a search would be a trip over the host link of its own.
+		*/
+		for (int i = tid; i < a.n_fix; i += kThreads)
+			fix_s[i] = a.fix[i];
+		__syncthreads();
 		/* the first entry not below c_lo (the same for every lane) */
 		while (len > 0) {
 			const int half = len / 2;
 
-			if (a.fix[at + half] < c_lo) {
+			if (fix_s[at + half] < c_lo) {
 				at += half + 1;
 				len -= half + 1;
 			} else {
 				len = half;
 			}
 		}
-		for (; at < a.n_fix && a.fix[at] < c_hi; at++) {
-			const int64_t c = a.fix[at];
-			double x = (NT && c < a.sum.keep_from) ? chunk_sum_lane<true>(a.sum, c, tid)
-			    : chunk_sum_lane<false>(a.sum, c, tid);
+		/* the run's chunks on the list, dealt to the four wavefronts in turn */
+		for (int i = at + (tid >> 6); i < a.n_fix && fix_s[i] < c_hi; i += kWaves) {
+			const int64_t c = fix_s[i];
+			const double x = (NT && c < a.sum.keep_from) ? chunk_sum_wave<true>(a.sum, c, tid & 63)
+			    : chunk_sum_wave<false>(a.sum, c, tid & 63);
 
-#pragma unroll
-			for (int off = 32; off > 0; off >>= 1)
-				x += __shfl_down(x, off, 64);
 			if ((tid & 63) == 0)
-				__hip_atomic_store(cells + c * kWaves + (tid >> 6),
-				    (unsigned long long)__double_as_longlong(x), __ATOMIC_RELAXED,
-				    __HIP_MEMORY_SCOPE_AGENT);
+				__hip_atomic_store(cells + c, (unsigned long long)__double_as_longlong(x),
+				    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 		}
 		__syncthreads();
 	}
@@ -1736,7 +1761,7 @@ int chunk_sums_count(int64_t n)
 }
 
 int launch_chunk_sums(hipStream_t st, const float *x, int64_t n, double *part, const int32_t *list,
-	int n_list)
+	int n_list, int beside)
 {
 	ChunkSumArgs a;
 	const int64_t n_chunks = chunk_sums_count(n);
@@ -1756,11 +1781,17 @@ int launch_chunk_sums(hipStream_t st, const float *x, int64_t n, double *part, c
 		a.keep_from = n_chunks > keep ? n_chunks - keep : 0;
 	}
 	if (list) {
-		grid = n_list;
+		grid = ((int64_t)n_list + kWaves - 1) / kWaves;		/* one wavefront per listed chunk */
 	} else {
-		grid = (int64_t)cu_count() * (sw().sumsq_per_cu ? sw().sumsq_per_cu : 2);
-		if (grid > n_chunks)
-			grid = n_chunks;
+		/*
+		** Workgroups per compute unit, resident as a whole.  Alone on the device eight are best
+		** (0.332 ms per call at 555M against 0.351 for two, 0.335 - 0.337 for 12 and 16); a sum that
+		** runs beside the caller's copy pieces leaves them room: with eight the unchanged caller's
+		** 555M step was 0.04 ms slower than with two.
+		*/
+		grid = (int64_t)cu_count() * (sw().sumsq_per_cu ? sw().sumsq_per_cu : beside ? 2 : 8);
+		if (grid > (n_chunks + kWaves - 1) / kWaves)
+			grid = (n_chunks + kWaves - 1) / kWaves;
 	}
 	if (grid < 1)
 		grid = 1;
@@ -1773,8 +1804,8 @@ int launch_chunk_sums(hipStream_t st, const float *x, int64_t n, double *part, c
 
 int launch_chunk_fold(hipStream_t st, const double *part, int64_t n, double *runs, StepState *state)
 {
-	const int64_t count = (int64_t)chunk_sums_count(n) * kWaves;
-	int64_t per = 2048;		/* partials per run: eight per lane */
+	const int64_t count = (int64_t)chunk_sums_count(n);
+	int64_t per = kChunkPer;
 	int64_t n_runs;
 
 	if (!part || !runs || !state || n <= 0)
@@ -1803,9 +1834,9 @@ static int chunk_finish_launch(hipStream_t st, const float *x, int64_t n, double
 	static ChunkFinishArgs a;	/* 3 KiB: off the stack; calls are serialised by the caller */
 	const int64_t n_chunks = chunk_sums_count(n);
 	const int64_t keep = (int64_t)keep_mb() * (1 << 20) / SumsqChunk<kF32>::kBytes;
-	int64_t per = 2048;
+	int64_t per = kChunkPer;
 
-	a.count = n_chunks * kWaves;
+	a.count = n_chunks;
 	while ((a.count + per - 1) / per > kChunkRuns)
 		per *= 2;
 	a.per = per;
@@ -1839,7 +1870,7 @@ static int chunk_finish_launch(hipStream_t st, const float *x, int64_t n, double
 static int chunk_finish_apart(hipStream_t st, const float *x, int64_t n, double *part, const int32_t *fix_dev,
 	int n_fix, double *runs, StepState *state)
 {
-	if (n_fix > 0 && launch_chunk_sums(st, x, n, part, fix_dev, n_fix) != 0)
+	if (n_fix > 0 && launch_chunk_sums(st, x, n, part, fix_dev, n_fix, 0) != 0)
 		return -1;
 	return launch_chunk_fold(st, part, n, runs, state);
 }

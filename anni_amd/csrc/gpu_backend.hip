@@ -381,7 +381,7 @@ static const void *g_pinned[PIN_SLOTS];
 static int g_pinned_n;
 
 /*
-** Scratch of the flat path's sum of squares: kWaves partial sums per 16 KiB chunk of the flat
+** Scratch of the flat path's sum of squares: one partial sum per 16 KiB chunk of the flat
 ** (grown when a longer flat comes), the sums of their runs, and the result in page-locked host
 ** memory, which the last kernel writes directly.
 */
@@ -436,7 +436,7 @@ static bool sum_scratch_locked(int64_t n)
 
 		/* nothing on the stream may still write the old block */
 		if (hipStreamSynchronize(g_stream) != hipSuccess
-		    || hipMalloc(&d, sizeof(double) * kWaves * (size_t)chunks) != hipSuccess) {
+		    || hipMalloc(&d, sizeof(double) * (size_t)chunks) != hipSuccess) {
 			(void)hipGetLastError();
 			return false;
 		}
@@ -632,7 +632,7 @@ static void early_sum_on_small_h2d_locked(const void *dev, size_t nbytes)
 			** of those whose partial sums are computed again once both have finished, so what the
 			** sum made of it is never used.
 			*/
-			if (launch_chunk_sums(g_side_stream, e.x, e.n, g_chunk_part, nullptr, 0) == 0) {
+			if (launch_chunk_sums(g_side_stream, e.x, e.n, g_chunk_part, nullptr, 0, 1) == 0) {
 				e.token = ++g_stamp_token;
 				hipLaunchKernelGGL(stamp_kernel, dim3(1), dim3(64), 0, g_side_stream, g_host_stamp + 1,
 				    e.token);
@@ -1680,7 +1680,7 @@ static int sumsq_enqueue_locked(const ann_real *d_x, int n, unsigned long long *
 		}
 	}
 	if (!early)
-		rc = launch_chunk_sums(g_stream, d_x, n, g_chunk_part, nullptr, 0);
+		rc = launch_chunk_sums(g_stream, d_x, n, g_chunk_part, nullptr, 0, 0);
 	if (rc == 0)
 		rc = launch_chunk_finish(g_stream, d_x, n, g_chunk_part, early ? e.dirty.data() : nullptr, fix_dev,
 		    early ? (int)e.dirty.size() : 0, g_chunk_runs, g_chunk_ticket, g_host_state, g_host_stamp,
