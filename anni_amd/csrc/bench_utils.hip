@@ -59,6 +59,33 @@ __global__ __launch_bounds__(kLanes) void copy16_kernel(void *dst, const void *s
 		((u32x4 *)dst)[i] = ((const u32x4 *)src)[i];
 }
 
+/*
+** The same copy in the update kernel's shape: one workgroup per 16 KiB, four 16-byte words per
+** lane in flight, the dispatcher handing the next piece to whichever compute unit falls free;
+** NT selects non-temporal loads and stores.  n16 is a multiple of 1024 here; the tail goes to
+** copy16_kernel.
+*/
+template <bool NT>
+__global__ __launch_bounds__(kLanes) void copy_tiled_kernel(void *dst, const void *src)
+{
+	typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+	const u32x4 *s = (const u32x4 *)src + (size_t)blockIdx.x * 1024 + threadIdx.x;
+	u32x4 *d = (u32x4 *)dst + (size_t)blockIdx.x * 1024 + threadIdx.x;
+	u32x4 w[4];
+
+	static_assert(kLanes == 256, "a piece is four words per lane");
+#pragma unroll
+	for (int u = 0; u < 4; u++)
+		w[u] = NT ? __builtin_nontemporal_load(s + u * 256) : s[u * 256];
+#pragma unroll
+	for (int u = 0; u < 4; u++) {
+		if (NT)
+			__builtin_nontemporal_store(w[u], d + u * 256);
+		else
+			d[u * 256] = w[u];
+	}
+}
+
 static int util_grid(int64_t items)
 {
 	int64_t g = (items + kLanes - 1) / kLanes;
@@ -200,6 +227,30 @@ int anni_copy_bytes(void *d_dst, const void *d_src, size_t nbytes)
 		return -1;
 	hipLaunchKernelGGL(copy16_kernel, dim3(util_grid((int64_t)(nbytes / 16))), dim3(kLanes), 0,
 	    (hipStream_t)anni_gpu_stream(), d_dst, d_src, nbytes / 16);
+	return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int anni_copy_bytes_tiled(void *d_dst, const void *d_src, size_t nbytes, int nontemporal)
+{
+	const size_t pieces = nbytes / 16384;
+	const size_t done = pieces * 16384;
+	hipStream_t st;
+
+	if (!d_dst || !d_src || nbytes == 0 || (nbytes & 15) || ((uintptr_t)d_dst & 15)
+	    || ((uintptr_t)d_src & 15) || pieces > 0x7fffffffu || !gpu_available())
+		return -1;
+	st = (hipStream_t)anni_gpu_stream();
+	if (pieces > 0) {
+		if (nontemporal)
+			hipLaunchKernelGGL((copy_tiled_kernel<true>), dim3((unsigned)pieces), dim3(kLanes), 0, st,
+			    d_dst, d_src);
+		else
+			hipLaunchKernelGGL((copy_tiled_kernel<false>), dim3((unsigned)pieces), dim3(kLanes), 0, st,
+			    d_dst, d_src);
+	}
+	if (done < nbytes)
+		hipLaunchKernelGGL(copy16_kernel, dim3(util_grid((int64_t)((nbytes - done) / 16))), dim3(kLanes), 0,
+		    st, (char *)d_dst + done, (const char *)d_src + done, (nbytes - done) / 16);
 	return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

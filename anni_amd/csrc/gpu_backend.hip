@@ -596,6 +596,18 @@ static bool early_sum_on(void)
 	return on == 1;
 }
 
+/* Work put on the second stream would not become part of a graph being recorded on the compute stream. */
+static bool compute_stream_is_recording(void)
+{
+	hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+
+	if (hipStreamIsCapturing(g_stream, &cs) != hipSuccess) {
+		(void)hipGetLastError();
+		return true;
+	}
+	return cs != hipStreamCaptureStatusNone;
+}
+
 static bool inside(const void *p, size_t nbytes, const void *base, size_t span)
 {
 	return base && (const char *)p >= (const char *)base
@@ -620,7 +632,8 @@ static void early_sum_on_small_h2d_locked(const void *dev, size_t nbytes)
 		e.seq_first = now;
 		e.began_clean = now == e.seq_at_sync;
 		if (!e.launched && e.shown >= 2 && e.began_clean && early_sum_on() && e.x
-		    && g_chunk_part && chunk_sums_count(e.n) <= g_chunk_cap && side_stream_locked()) {
+		    && g_chunk_part && chunk_sums_count(e.n) <= g_chunk_cap && !compute_stream_is_recording()
+		    && side_stream_locked()) {
 			/*
 			** On a stream of its own, so that the uploads that follow run beside it instead of
 			** queueing up behind it.  No event ties the two streams together (recording and
@@ -1799,7 +1812,8 @@ int gpu_adam_step_dev_bf16(ann_real *d_param, void *d_param_bf16, ann_real *d_gr
 			if (v.built && v.shown >= 2 && !pending && before == g_early.seq_at_sync
 			    && d_param == v.learned_p && n == v.learned_n && vectors_first_on()
 			    && v.built_backwards == update_walks_backwards()
-			    && (g_host_stamp || sum_scratch_locked(1)) && side_stream_locked()) {
+			    && (g_host_stamp || sum_scratch_locked(1)) && !compute_stream_is_recording()
+			    && side_stream_locked()) {
 				rc = launch_update_tiles(g_stream, f, c, grad_scale, norm, v.order + v.k_first,
 				    v.n_tiles - v.k_first);
 				if (rc == 0) {

@@ -142,6 +142,7 @@ _BENCH_PROTOS = {
     "anni_fill_normal_f32": (C.c_int, [C.c_void_p, C.c_int64, C.c_uint64, C.c_uint64,
                                        C.c_float, C.c_float]),
     "anni_copy_bytes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "anni_copy_bytes_tiled": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]),
     "anni_fold_guard_stats": (C.c_int, [C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "anni_early_sum_stats": (C.c_int, [C.POINTER(C.c_long), C.POINTER(C.c_long)]),
     "anni_vectors_first_stats": (C.c_int, [C.POINTER(C.c_long), C.POINTER(C.c_long)]),

@@ -637,8 +637,10 @@ def sections_leg(L, n=555848096, region_gib=16):
 
 def ceilings(L, nbytes=8 << 30):
     """What this box delivers to the simplest kernels of the library: write-only (fill), copy
-    (16-byte vectors, read + write) and read-only (the sum of squares), for comparison with the
-    update's mixed stream."""
+    (16-byte vectors, read + write: the grid-stride loop of the counter calibration, and one
+    workgroup per 16 KiB as the update does it, with and without non-temporal hints) and read-only
+    (the sum of squares), for comparison with the update's mixed stream.  The two blocks come from
+    gpu_malloc's two pools, i.e. from different memory sections, like the halves of an arena."""
     a, b = L.gpu_malloc(nbytes), L.gpu_malloc(nbytes)
     assert a and b
     assert L.gpu_memset(a, 1, nbytes) == 0 and L.gpu_memset(b, 0, nbytes) == 0
@@ -658,6 +660,10 @@ def ceilings(L, nbytes=8 << 30):
            "write_only_GBps": round(nbytes / timed(lambda: L.gpu_memset(b, 3, nbytes)) / 1e9, 1),
            "copy_read_plus_write_GBps":
                round(2 * nbytes / timed(lambda: L.anni_copy_bytes(b, a, nbytes)) / 1e9, 1),
+           "copy_in_the_updates_shape_GBps":
+               round(2 * nbytes / timed(lambda: L.anni_copy_bytes_tiled(b, a, nbytes, 0)) / 1e9, 1),
+           "copy_in_the_updates_shape_nontemporal_GBps":
+               round(2 * nbytes / timed(lambda: L.anni_copy_bytes_tiled(b, a, nbytes, 1)) / 1e9, 1),
            "read_only_GBps":
                round(n * 4 / timed(lambda: L.gpu_grad_sumsq(a, n, C.byref(ss))) / 1e9, 1)}
     L.gpu_free(a)

@@ -35,6 +35,12 @@ int	anni_fill_normal_f32(float *d_x, int64_t n, uint64_t seed, uint64_t stream,
 /* Plain 16-byte-vector copy kernel of nbytes (a multiple of 16, 16-byte aligned): reads and writes exactly nbytes. */
 int	anni_copy_bytes(void *d_dst, const void *d_src, size_t nbytes);
 /*
+** The same copy in the shape of the update kernel (one workgroup per 16 KiB, four 16-byte words
+** per lane in flight, as many workgroups as pieces); nontemporal != 0 uses non-temporal loads and
+** stores.  For `bench.py --ceilings`: what a copy shaped like the update reaches on this device.
+*/
+int	anni_copy_bytes_tiled(void *d_dst, const void *d_src, size_t nbytes, int nontemporal);
+/*
 ** Reads the kernels' tuning switches (ANNI_TILES_PER_WG, ANNI_KEEP_MB, ANNI_REVERSE, ANNI_PIPE,
 ** ANNI_NT, ANNI_BLOCKS_PER_CU) from the environment again; without this call they are read once,
 ** on first use.  For sweeps that compare settings on one arena inside one process (two
