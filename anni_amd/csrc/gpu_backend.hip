@@ -460,9 +460,9 @@ static bool sum_scratch_locked(int64_t n)
 ** pass; the caller synchronises before it begins, :539).  So once the caller has shown the pattern
 ** twice in a row -- since the last synchronisation nothing but small uploads, then gpu_grad_sumsq
 ** of the same flat -- the next first small upload into that flat or into the registered parameter
-** flat (gpu_adam_set_bf16_flat) puts the chunk sums of the whole gradient flat on the stream ahead
-** of the upload.  The chunks that small uploads write afterwards are noted; gpu_grad_sumsq then
-** recomputes the partial sums of just those and folds.  The sum is a function of the flat's
+** flat (gpu_adam_set_bf16_flat) launches the chunk sums of the whole gradient flat on a second
+** stream, where they run beside the uploads.  The chunks that small uploads write afterwards are
+** noted; gpu_grad_sumsq then recomputes the partial sums of just those and folds.  The sum is a function of the flat's
 ** contents alone (adam_kernels.hip, chunk_sums_kernel), so the result has the bits of a sum begun
 ** when it was asked for.
 **
@@ -659,7 +659,7 @@ static void early_sum_on_small_h2d_locked(const void *dev, size_t nbytes)
 	}
 	if (e.launched && in_grad) {
 		const size_t off = (size_t)((const char *)dev - (const char *)e.x);
-		const size_t chunk = 16384;
+		const size_t chunk = 16384;	/* the unit of launch_chunk_sums' partial sums (adam_kernels.h) */
 
 		for (size_t c = off / chunk; c <= (off + nbytes - 1) / chunk; c++) {
 			if (e.dirty.size() >= kEarlyDirtyMax) {
