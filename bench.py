@@ -250,8 +250,10 @@ def placement_cost_leg(L):
     return out
 
 
-def cpu_baselines(size_name, norm_bpp, upd_bpp, budget_s):
-    """The step on the host cores of this box: (multithreaded port, single-thread reference)."""
+def cpu_baselines(size_name, norm_bpp, upd_bpp, budget_s, full=False):
+    """The step on the host cores of this box: (multithreaded port, single-thread reference).
+    full: the multithreaded leg runs on the workload's whole parameter count instead of a
+    48 Mi sample (about 10 GB of host memory and half a minute more at 555M)."""
     from anni_amd import layout
     from oracle import binding as ob
     ob.lib()
@@ -266,7 +268,7 @@ def cpu_baselines(size_name, norm_bpp, upd_bpp, budget_s):
         return p, g0
 
     # multithreaded restatement, SoA, all cores; norm by ordered partials
-    n = min(n_full, 48 << 20)
+    n = n_full if full else min(n_full, 48 << 20)
     p, g0 = sample(n)
     m = np.zeros(n, np.float32)
     v = np.zeros(n, np.float32)
@@ -289,7 +291,7 @@ def cpu_baselines(size_name, norm_bpp, upd_bpp, budget_s):
     mt_out = {
         "value": round(n * bpp / mt / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
         "simd": simd,
-        "sample": "first %d of %d params of the workload, %d timed steps (median), fp32 state, "
+        "sample": ("all" if n == n_full else "first") + " %d of %d params of the workload, %d timed steps (median), fp32 state, "
                   "clip 1.0 + decay 0.1, OpenMP over %d threads, %s build (gcc -O3 auto-vectorised, "
                   "no FMA contraction: bit-identical to the serial loop)"
                   % (n, n_full, len(times), threads, simd),
@@ -697,6 +699,8 @@ def main():
     ap.add_argument("--layout", default="auto", choices=["auto", "compact", "split"],
                     help="arena layout (split: two allocations in different 96 GiB sections of device memory)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
+    ap.add_argument("--cpu-full", action="store_true",
+                    help="time the multithreaded host baseline on the whole parameter set, not a sample")
     ap.add_argument("--no-legs", action="store_true",
                     help="skip the side legs of the headline workload (compact layout, 185m)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
@@ -938,7 +942,7 @@ def main():
             "separate_passes_would_move_bytes": 9 * fp8_elems + 4 * pack_elems,
             "fused_moves_bytes": extra_bytes}
     if not a.no_cpu:
-        mt_out, serial_out = cpu_baselines(size, norm_bpp, upd_bpp, a.cpu_budget)
+        mt_out, serial_out = cpu_baselines(size, norm_bpp, upd_bpp, a.cpu_budget, a.cpu_full)
         out["cpu_baseline"] = mt_out
         out["cpu_reference_serial"] = serial_out
         out["gpu_over_cpu"] = round(step_gbps / mt_out["value"], 1)
