@@ -157,6 +157,7 @@ int	launch_update_tiles(hipStream_t st, const Flat &f, const StepConsts &c, doub
 ** The sum is a function of x alone: partials recomputed for some chunks after their elements
 ** changed give the bits a pass over the whole flat would.
 */
+constexpr size_t kSumChunkBytes = 16384;	/* a chunk; callers that track rewritten chunks count in these */
 constexpr int kChunkRuns = 1024;
 constexpr int kChunkPer = 512;		/* two partials per lane of the workgroup that folds a run */
 int	chunk_sums_count(int64_t n);

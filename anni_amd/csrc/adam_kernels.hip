@@ -1753,6 +1753,8 @@ int launch_sumsq(hipStream_t st, const Flat &f, double grad_scale, double *parti
 	return sumsq_launch(st, f, grad_scale, partials, n_partials, fin, sw().fold_fence);
 }
 
+static_assert(SumsqChunk<kF32>::kBytes == (int64_t)kSumChunkBytes, "callers note rewritten chunks in these units");
+
 int chunk_sums_count(int64_t n)
 {
 	const int64_t c = (n + SumsqChunk<kF32>::kElems - 1) / SumsqChunk<kF32>::kElems;
@@ -1831,7 +1833,7 @@ static int chunk_finish_launch(hipStream_t st, const float *x, int64_t n, double
 	int n_fix, double *runs, unsigned int *ticket, StepState *state, unsigned long long *stamp,
 	unsigned long long token)
 {
-	static ChunkFinishArgs a;	/* 3 KiB: off the stack; calls are serialised by the caller */
+	ChunkFinishArgs a;
 	const int64_t n_chunks = chunk_sums_count(n);
 	const int64_t keep = (int64_t)keep_mb() * (1 << 20) / SumsqChunk<kF32>::kBytes;
 	int64_t per = kChunkPer;

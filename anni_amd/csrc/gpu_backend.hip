@@ -659,7 +659,7 @@ static void early_sum_on_small_h2d_locked(const void *dev, size_t nbytes)
 	}
 	if (e.launched && in_grad) {
 		const size_t off = (size_t)((const char *)dev - (const char *)e.x);
-		const size_t chunk = 16384;	/* the unit of launch_chunk_sums' partial sums (adam_kernels.h) */
+		const size_t chunk = kSumChunkBytes;
 
 		for (size_t c = off / chunk; c <= (off + nbytes - 1) / chunk; c++) {
 			if (e.dirty.size() >= kEarlyDirtyMax) {
