@@ -772,6 +772,7 @@ static void vf_side_wait_locked(void)
 	if (!stamp_wait(g_host_stamp + 1, v.token))
 		(void)hip_ok_locked(hipStreamSynchronize(g_side_stream), "side stream");
 	v.side_pending = false;
+	v.active = false;	/* whatever is asked for from here on is copied the ordinary way */
 	g_vf_side_pending.store(0, std::memory_order_release);
 	for (const Delivery &d : v.deliver)
 		memcpy(d.host, v.stage + d.stage_off, d.nbytes);
@@ -1804,6 +1805,9 @@ int gpu_adam_step_dev_bf16(ann_real *d_param, void *d_param_bf16, ann_real *d_gr
 			std::lock_guard<std::mutex> lk(g_mu);
 			VectorsFirst &v = g_vf;
 			bool split = false;
+
+			v.active = false;	/* read-backs are matched only after an update that was split */
+			v.deliver.clear();
 
 			/*
 			** "The vectors first": only with the list built for this very flat, and only when the

@@ -906,3 +906,146 @@ def test_vectors_first_split_update_serves_the_read_backs_and_leaves_no_tile_out
     assert counters()[0] == 5
     gpu.gpu_set_compute_prec(0)
     gpu.gpu_adam_set_weight_decay(0.0)
+
+
+@pytest.mark.parametrize("seed", list(range(1, 11)))
+def test_random_call_sequences_against_a_host_model(gpu, oracle, seed):
+    """The flat entry points under call sequences nobody wrote by hand: the caller's regular step
+    (which, repeated, brings in the sum begun early and the split update) mixed at random with
+    everything that must make the backend drop what it began -- large and small uploads, fills,
+    read-backs of other places, extra sums, extra synchronisations, uploads that overlap -- against
+    a model kept on the host: every sum within 1e-10 of the exact one and equal to a second call's,
+    every read-back equal to the model at the time it was asked for, and p, g, m, v and the twins
+    equal to the model's bits after every round."""
+    rng = np.random.default_rng(1000 + seed)
+    n = 4096 * 290 + 1000 + seed
+    S = FlatState(gpu, n, seed=seed)
+    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, threads=8)
+    gpu.gpu_set_compute_prec(1)
+    gpu.gpu_adam_set_bf16_flat(S.dt.ptr, S.dp.ptr, n)
+    S.twin[:] = oracle.bf16_rne(S.p)
+    assert gpu.gpu_adam_seed_bf16_flat(S.dt.ptr, S.dp.ptr, n) == 0
+    flats = {"p": (S.dp, S.p), "g": (S.dg, S.g), "m": (S.dm, S.m), "v": (S.dv, S.v)}
+    vecs = [(int(o), int(c)) for o, c in zip(rng.integers(0, n - 5000, 9), rng.integers(1, 5000, 9))]
+    pending = []                                         # read-backs asked for: (buffer, expected)
+    keep = []
+    t = [0]
+
+    def upload(name, off, values):
+        buf, host = flats[name]
+        a = np.ascontiguousarray(values, dtype=np.float32)
+        keep.append(a)
+        host[off:off + a.size] = a
+        assert gpu.gpu_memcpy_h2d(buf.ptr + 4 * off, a.ctypes.data, 4 * a.size) == 0
+
+    def read_back(name, off, cnt):
+        buf, host = flats[name]
+        out = np.full(cnt, np.nan, np.float32)
+        assert gpu.gpu_memcpy_d2h_async(out.ctypes.data, buf.ptr + 4 * off, 4 * cnt) == 0
+        pending.append((out, host[off:off + cnt].copy()))
+
+    def sync(which):
+        if which:
+            assert gpu.gpu_stream_sync() == 0
+        else:
+            gpu.gpu_device_sync()
+        for out, want in pending:
+            assert same_bits(out, want)
+        pending.clear()
+
+    def sumsq():
+        out = C.c_double(0)
+        assert gpu.gpu_grad_sumsq(S.dg.ptr, n, C.byref(out)) == 0
+        for o, want in pending:                          # the call implies a synchronisation
+            assert same_bits(o, want)
+        pending.clear()
+        want = oracle.sumsq(S.g, threads=4)
+        assert abs(out.value - want) <= 1e-10 * want, (out.value, want)
+        return out.value
+
+    def update(gs):
+        t[0] += 1
+        lr = 1e-3 / t[0]
+        gpu.gpu_adam_set_weight_decay(0.1)
+        assert gpu.gpu_adam_step_dev_bf16(S.dp.ptr, S.dt.ptr, S.dg.ptr, S.dm.ptr, S.dv.ptr, n, lr,
+                                          0.9, 0.95, 1e-8, t[0], gs) == 0
+        O.step(S.p, S.g, S.m, S.v, lr, gs, twin=S.twin)
+
+    def disturbance():
+        k = int(rng.integers(0, 11))
+        if k == 0:
+            off = int(rng.integers(0, n - 400000))
+            upload("g", off, rng.standard_normal(300000) * 1e-3)          # more than 1 MiB: an ordinary copy
+        elif k == 1:
+            off, cnt = int(rng.integers(0, n - 3000)), int(rng.integers(1, 3000))
+            name = "pg"[int(rng.integers(0, 2))]
+            assert gpu.gpu_memset(flats[name][0].ptr + 4 * off, 0, 4 * cnt) == 0
+            flats[name][1][off:off + cnt] = 0.0
+        elif k == 2:
+            read_back("pgmv"[int(rng.integers(0, 4))], int(rng.integers(0, n - 2000)), int(rng.integers(1, 2000)))
+        elif k == 3:
+            assert sumsq() == sumsq()
+        elif k == 4:
+            sync(int(rng.integers(0, 2)))
+        elif k == 5:
+            off = int(rng.integers(0, n - 300))
+            for _ in range(3):                           # the same place three times: the last one wins
+                upload("pg"[int(rng.integers(0, 2))], off, rng.standard_normal(200) * 1e-3)
+        elif k == 6:
+            update(float(rng.random()) + 0.1)            # an update nobody announced
+        elif k == 7:
+            out = np.empty(1000, np.float32)
+            off = int(rng.integers(0, n - 1000))
+            assert gpu.gpu_memcpy_d2h(out.ctypes.data, S.dp.ptr + 4 * off, 4000) == 0
+            assert same_bits(out, S.p[off:off + 1000])
+            for o, want in pending:
+                assert same_bits(o, want)
+            pending.clear()
+        elif k == 8:
+            out = C.c_double(0)                          # the sum of another flat
+            assert gpu.gpu_grad_sumsq(S.dp.ptr, n, C.byref(out)) == 0
+            want = oracle.sumsq(S.p, threads=4)
+            assert abs(out.value - want) <= 1e-10 * want
+            for o, w in pending:
+                assert same_bits(o, w)
+            pending.clear()
+        elif k == 9:
+            gpu.anni_gpu_flush()                         # a caller announcing work of its own on the stream
+        # k == 10: nothing
+
+    def regular_step(noise):
+        """adam_step_gpu's order of calls; `noise` = chance of a disturbance at each of its joints."""
+        S.new_grad(1e-3 * (1 + t[0] % 3))                # "the backward pass": a large upload
+        sync(0)
+        for off, cnt in vecs:
+            if rng.random() < noise:
+                disturbance()
+            upload("p", off, S.p[off:off + cnt] * np.float32(1.0))
+            upload("g", off, rng.standard_normal(cnt) * 1e-3)
+        if rng.random() < noise:
+            disturbance()
+        ss = sumsq()
+        if rng.random() < noise:
+            disturbance()
+        gs = 1.0 / (math.sqrt(n) * 1e-3) * (1.7 if t[0] % 2 else 0.6)
+        norm = math.sqrt(oracle.sumsq(S.g, threads=4)) * gs if noise else math.sqrt(ss) * gs
+        update(gs / norm if norm > 1.0 else gs)
+        for off, cnt in vecs:
+            if rng.random() < noise:
+                disturbance()
+            read_back("p", off, cnt)
+        sync(1)
+        p, m, v, g, tw = S.fetch()
+        assert same_bits(p, S.p) and same_bits(m, S.m) and same_bits(v, S.v) and same_bits(g, S.g), t[0]
+        assert (tw == S.twin).all(), t[0]
+    for rnd in range(6):
+        for _ in range(4):
+            regular_step(0.0)                            # long enough for both patterns to be learned and used
+        for _ in range(4):
+            regular_step(0.3 if rnd % 3 == 2 else 0.08)
+    early, dropped = C.c_long(0), C.c_long(0)
+    gpu.anni_early_sum_stats(C.byref(early), C.byref(dropped))
+    assert early.value > 0
+    gpu.gpu_adam_set_bf16_flat(None, None, 0)
+    gpu.gpu_set_compute_prec(0)
+    gpu.gpu_adam_set_weight_decay(0.0)
