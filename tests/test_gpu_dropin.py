@@ -972,7 +972,7 @@ def test_random_call_sequences_against_a_host_model(gpu, oracle, seed):
         O.step(S.p, S.g, S.m, S.v, lr, gs, twin=S.twin)
 
     def disturbance():
-        k = int(rng.integers(0, 11))
+        k = int(rng.integers(0, 12))
         if k == 0:
             off = int(rng.integers(0, n - 400000))
             upload("g", off, rng.standard_normal(300000) * 1e-3)          # more than 1 MiB: an ordinary copy
@@ -1011,7 +1011,10 @@ def test_random_call_sequences_against_a_host_model(gpu, oracle, seed):
             pending.clear()
         elif k == 9:
             gpu.anni_gpu_flush()                         # a caller announcing work of its own on the stream
-        # k == 10: nothing
+        elif k == 10 and not pending:
+            S.dg.free()                                  # the gradient flat freed and allocated anew
+            S.dg = dev(gpu, S.g)                         # (the driver may hand out the same address)
+            flats["g"] = (S.dg, S.g)
 
     def regular_step(noise):
         """adam_step_gpu's order of calls; `noise` = chance of a disturbance at each of its joints."""
