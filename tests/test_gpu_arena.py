@@ -761,3 +761,89 @@ def test_op_prof_times_the_arena_steps_launches(gpu):
     for name, got in per.items():
         assert sum(c for _ms, c in got) == 3, (name, got)
         assert all(0.0 < ms < 50.0 for ms, _c in got), (name, got)
+
+
+@pytest.mark.parametrize("seed,mode", [(1, "f32"), (2, "bf16"), (3, "f32"), (4, "bf16"), (5, "f32"), (6, "bf16")])
+def test_random_sequences_of_arena_calls_against_the_oracle(gpu, oracle, seed, mode):
+    """The arena's entry points in an order nobody wrote by hand: steps (clipped and not, with a NaN
+    now and then), the moments sent to the host and brought back, gradient slots switched, the
+    gradients cleared, slices of the optimizer block exported and imported -- against the oracle,
+    bit for bit under the device's sum, after every call that changes state."""
+    narrow = mode == "bf16"
+    rng = np.random.default_rng(7000 + seed)
+    tensors = [(4096 * 70 + 13, 3), (333, 0), (4096 * 20, 3), (1, 1), (50000, 2), (4096 * 45 + 4000, 3), (77, 0)]
+    opt = make(gpu, tensors, grad_type=0, moment_type=1 if narrow else 0, grad_slots=2, beta2=0.95,
+               weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True)
+    n = opt.n
+    P = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    opt.upload("param", P)
+    opt.seed_twins()
+    TW = oracle.bf16_rne(P)
+    M = np.zeros(n, np.uint16 if narrow else np.float32)
+    V = np.zeros(n, np.uint16 if narrow else np.float32)
+    O = oracle.Oracle(n, beta2=0.95, weight_decay=0.1, grad_clip=1.0, skip_nonfinite=True,
+                      moment_type=oracle.BF16 if narrow else oracle.F32, tensors=oracle_tensors(opt), threads=8)
+    wide = (lambda a: oracle.bf16_widen(a)) if narrow else (lambda a: a)
+    mask = twin_mask(opt)
+    unit = 1.0 / (np.sqrt(n) * 1e-3)
+    parked = [False]
+    slot = [0]
+    G = [np.zeros(n, np.float32), np.zeros(n, np.float32)]     # what each gradient slot holds
+
+    def check_state():
+        assert same_bits(opt.download("param"), P)
+        assert (opt.download("twin")[mask] == TW[mask]).all()
+        assert same_bits(opt.download("grad"), G[slot[0]])
+        if parked[0]:
+            assert gpu.anni_adam_mv_on_device(opt.h) == 0
+            first = int(rng.integers(0, n - 3000))
+            pairs = opt.export_mv(first, 3000)
+            assert same_bits(pairs[:, 0].copy(), wide(M[first:first + 3000]))
+            assert same_bits(pairs[:, 1].copy(), wide(V[first:first + 3000]))
+        else:
+            gm, gv = opt.download("m"), opt.download("v")
+            assert (gm.view(M.dtype) == M).all() and (gv.view(V.dtype) == V).all()
+
+    def step(kind):
+        g = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+        if kind == "nan":
+            g[int(rng.integers(0, n))] = np.nan
+        if kind != "cleared":
+            opt.upload("grad", g)
+            G[slot[0]][:] = g
+        gs = unit * (1.7 if rng.random() < 0.5 else 0.6)
+        lr = 1e-3 * float(rng.random() + 0.1)
+        assert opt.step_scaled(lr, gs) == 0
+        st = opt.sync_stats()
+        assert st.last_skipped == (1 if kind == "nan" else 0)
+        O.step(P, G[slot[0]], M, V, lr, gs, twin=TW, sumsq_override=st.last_sumsq)
+    for _ in range(40):
+        k = int(rng.integers(0, 10))
+        if k <= 3:
+            step("plain")
+        elif k == 4:
+            step("nan")
+        elif k == 5:
+            parked[0] = not parked[0]
+            assert gpu.anni_adam_set_offload(opt.h, 1 if parked[0] else 0) == 0, gpu.gpu_debug_last_error()
+        elif k == 6:
+            slot[0] ^= 1
+            opt.bind_grad(opt.grad_slot(slot[0]))
+        elif k == 7:
+            assert opt.zero_grad() in (0, None)
+            G[slot[0]][:] = 0.0
+            step("cleared")
+        elif k == 8:
+            first, cnt = int(rng.integers(0, n - 5000)), int(rng.integers(1, 5000))
+            pairs = (rng.standard_normal((cnt, 2)) * 1e-4).astype(np.float32)
+            pairs[:, 1] = np.abs(pairs[:, 1])
+            opt.import_mv(pairs, first)
+            M[first:first + cnt] = oracle.bf16_rne(pairs[:, 0].copy()) if narrow else pairs[:, 0]
+            V[first:first + cnt] = oracle.bf16_rne(pairs[:, 1].copy()) if narrow else pairs[:, 1]
+        else:
+            first, cnt = int(rng.integers(0, n - 5000)), int(rng.integers(1, 5000))
+            pairs = opt.export_mv(first, cnt)
+            assert same_bits(pairs[:, 0].copy(), wide(M[first:first + cnt]))
+            assert same_bits(pairs[:, 1].copy(), wide(V[first:first + cnt]))
+        check_state()
+    opt.free()
