@@ -368,10 +368,13 @@ def reference_caller_leg(L, size="185m", call_trace=False):
     n = M.n
     vec_bytes = 4 * sum(cnt for _off, cnt, is_mat in M.segs() if not is_mat)
     rng = np.random.default_rng(1)
-    g = rng.standard_normal(n, dtype=np.float32) * np.float32(1e-3)
+    # 16 Mi normal deviates, repeated: what the step costs does not depend on the values, and
+    # drawing 5.6e8 of them would take longer than all the timed steps together
+    block = rng.standard_normal(1 << 24, dtype=np.float32) * np.float32(1e-3)
+    g = np.tile(block, -(-n // block.size))[:n]
     unit = 1.0 / (math.sqrt(n) * 1e-3)
     times = []
-    last = 13
+    last = 12
     for t in range(1, last + 1):
         M.set_grads(g)
         L.gpu_device_sync()
@@ -689,6 +692,16 @@ def copy_calibration(L, nbytes):
                       "GBps_read_plus_write": round(2 * nbytes / ms / 1e6, 1)}))
 
 
+_LAP = [time.perf_counter()]
+
+
+def lap(what):
+    """Where the run's wall clock goes, on stderr (the result line on stdout stays one JSON object)."""
+    now = time.perf_counter()
+    print("[bench] %-32s %6.1f s" % (what, now - _LAP[0]), file=sys.stderr, flush=True)
+    _LAP[0] = now
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -941,11 +954,13 @@ def main():
             "fp8_twin_elems": fp8_elems, "packed_elems": pack_elems,
             "separate_passes_would_move_bytes": 9 * fp8_elems + 4 * pack_elems,
             "fused_moves_bytes": extra_bytes}
+    lap("headline workload on the GPU")
     if not a.no_cpu:
         mt_out, serial_out = cpu_baselines(size, norm_bpp, upd_bpp, a.cpu_budget, a.cpu_full)
         out["cpu_baseline"] = mt_out
         out["cpu_reference_serial"] = serial_out
         out["gpu_over_cpu"] = round(step_gbps / mt_out["value"], 1)
+        lap("host baselines")
     opt.free()
     opt = None
     if not a.no_cpu and not a.no_legs:
@@ -955,6 +970,7 @@ def main():
                 ref_leg = reference_caller_leg(L, size)
                 if ref_leg:
                     out["reference_caller_" + size] = ref_leg
+                lap("reference caller " + size)
         except Exception as e:                      # the checker must never sink the bench line
             out["reference_caller_error"] = repr(e)
     if a.workload == "555m" and not a.derived and not a.no_legs:
@@ -962,9 +978,11 @@ def main():
         # metric names, each on an arena of its own after the one before it was freed
         try:
             out["layout_compact"] = short_leg(L, "555m", "compact")
+            lap("one-allocation leg")
             out["workloads"] = {}
             for w in ("185m", "555m-bf16", "1p4b-fp8"):
                 out["workloads"][w] = short_leg(L, w, "auto")
+                lap("workload " + w)
         except Exception as e:                      # a side leg must never sink the bench line
             out["side_legs_error"] = repr(e)
     if a.ref_jsonl:
