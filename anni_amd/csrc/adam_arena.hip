@@ -1511,6 +1511,8 @@ long anni_hook_counter(const char *name)
 		return used;
 	if (strcmp(name, "early_sum_dropped") == 0)
 		return dropped;
+	if (strcmp(name, "second_stream") == 0)
+		return second_stream_state();
 	if (strcmp(name, "vectors_first_steps") == 0 || strcmp(name, "vectors_first_served") == 0) {
 		long steps = 0, served = 0;
 

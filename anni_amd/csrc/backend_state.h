@@ -40,6 +40,8 @@ hipError_t	device_alloc(void **p, size_t nbytes);
 void		early_sum_stats(long *used, long *dropped);
 /* Steps whose small read-backs were served by a split update (gpu_backend.hip, "the vectors first"), and how many read-backs. */
 void		vectors_first_stats(long *steps, long *served);
+/* The search for a stream that runs beside the compute stream: -1 not made yet, 0 none found, 1 found. */
+int		second_stream_state(void);
 
 /*
 ** ANN_OP_PROF=1 (num/gpu_cuda.cu:3205-3409): an event pair around an operation of the optimizer

@@ -277,6 +277,11 @@ int anni_early_sum_stats(long *used, long *dropped)
 	return 0;
 }
 
+int anni_second_stream_state(void)
+{
+	return (int)anni_hook_counter("second_stream");
+}
+
 int anni_vectors_first_stats(long *steps, long *served)
 {
 	if (steps)

@@ -1876,6 +1876,16 @@ void early_sum_stats(long *used, long *dropped)
 		*dropped = g_early.dropped;
 }
 
+/* -1: no second stream has been looked for yet; 0: none runs beside the compute stream; 1: found. */
+int second_stream_state(void)
+{
+	std::lock_guard<std::mutex> lk(g_mu);
+
+	if (g_side_for != g_stream)
+		return -1;
+	return g_side_stream ? 1 : 0;
+}
+
 /* Steps whose read-backs were served by a split update, and how many read-backs that were. */
 void vectors_first_stats(long *steps, long *served)
 {

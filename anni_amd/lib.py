@@ -146,6 +146,7 @@ _BENCH_PROTOS = {
     "anni_fold_guard_stats": (C.c_int, [C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "anni_early_sum_stats": (C.c_int, [C.POINTER(C.c_long), C.POINTER(C.c_long)]),
     "anni_vectors_first_stats": (C.c_int, [C.POINTER(C.c_long), C.POINTER(C.c_long)]),
+    "anni_second_stream_state": (C.c_int, []),
 }
 
 _lib = None

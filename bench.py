@@ -408,7 +408,9 @@ def reference_caller_leg(L, size="185m", call_trace=False):
            "sums_begun_at_the_first_upload_and_used": used.value - used0.value,
            "sums_begun_early_and_dropped": dropped.value - dropped0.value,
            "steps_with_the_vectors_updated_and_read_back_first": vsteps.value - vsteps0.value,
-           "read_backs_served_that_way": vserved.value - vserved0.value}
+           "read_backs_served_that_way": vserved.value - vserved0.value,
+           "a_stream_that_runs_beside_the_compute_stream_was_found":
+               {-1: "not looked for", 0: "no", 1: "yes"}[L.anni_second_stream_state()]}
     if events:
         out["call_trace_of_the_last_step"] = call_timeline(events, times[-1])
     return out

