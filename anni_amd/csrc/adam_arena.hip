@@ -855,8 +855,14 @@ static int mv_bring(anni_adam *opt)
 	}
 	st = compute_stream();
 	if (!hip_ok(hipMemcpyAsync(opt->d_m, pv->h_m, pv->z.mv_bytes, hipMemcpyHostToDevice, st), "offload h2d")
-	    || !hip_ok(hipMemcpyAsync(opt->d_v, pv->h_v, pv->z.mv_bytes, hipMemcpyHostToDevice, st), "offload h2d"))
+	    || !hip_ok(hipMemcpyAsync(opt->d_v, pv->h_v, pv->z.mv_bytes, hipMemcpyHostToDevice, st), "offload h2d")) {
+		/* the host copies stay the valid ones: nothing half-filled may pass for the moments */
+		(void)sync_stream_and_deliver();
+		gpu_free(opt->d_m);
+		gpu_free(opt->d_v);
+		opt->d_m = opt->d_v = nullptr;
 		return -1;
+	}
 	return 0;
 }
 
